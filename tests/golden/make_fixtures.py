@@ -1,0 +1,157 @@
+"""Writes the golden vectors under tests/golden/ by running the reference itself.
+
+Run once, in a container that has the reference checkout, on CPU:
+
+    python tests/golden/make_fixtures.py [/root/reference]
+
+It imports optimi from that path, drives its optimizer classes with
+``triton=False, foreach=False`` (the PyTorch for-loop path) on small seeded
+tensors, and stores inputs (initial params, the gradient of every step) and
+outputs (params and every state tensor after selected steps) as ``.npz``
+files.  bf16 tensors are stored as their raw 16-bit patterns (uint16).
+
+The fixtures are data only; the tests read them with ``numpy.load`` and never
+need the reference.  Each case is described in ``CASES`` below, which the tests
+import to know the hyper-parameters of a fixture.
+"""
+
+from __future__ import annotations
+
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+# tensor shapes of every case: one 2-D tensor whose size is not a multiple of any
+# vector width, one small 1-D tensor
+SHAPES = [(33, 37), (256,)]
+SNAP_STEPS = (1, 3)  # besides the last step: lerp uses its large-weight branch at t<=2
+
+ADAMW = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
+LION = dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1)
+SADAMW = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
+ADAN = dict(lr=1e-3, betas=(0.98, 0.92, 0.99), eps=1e-8, weight_decay=2e-2)
+
+# name -> (class name, kwargs, dtype, mode, n_steps)
+# mode "group": optimizer.step() on the whole list.
+# mode "release": per-tensor step(param=p) in reverse order, accumulate-only on
+#                 micro-steps where (i+1) % 4 != 0 (optimizer accumulation).
+CASES = {
+    "adam_fp32_l2": ("Adam", dict(ADAMW, decouple_wd=False), "float32", "group", 10),
+    "adam_fp32_nowd": ("Adam", dict(ADAMW, weight_decay=0.0), "float32", "group", 10),
+    "adamw_fp32": ("AdamW", dict(ADAMW), "float32", "group", 10),
+    "adamw_bf16_kahan": ("AdamW", dict(ADAMW), "bfloat16", "group", 10),
+    "adamw_bf16_kahan_bigwd": ("AdamW", dict(ADAMW, lr=1e-2, weight_decay=1.0), "bfloat16", "group", 10),
+    "adamw_bf16_kahan_declr": ("AdamW", dict(ADAMW, weight_decay=1e-5, decouple_lr=True), "bfloat16", "group", 10),
+    "adamw_bf16_plain": ("AdamW", dict(ADAMW, kahan_sum=False), "bfloat16", "group", 10),
+    "adam_bf16_kahan_l2": ("Adam", dict(ADAMW, decouple_wd=False), "bfloat16", "group", 10),
+    "lion_fp32": ("Lion", dict(LION), "float32", "group", 10),
+    "lion_bf16_kahan": ("Lion", dict(LION), "bfloat16", "group", 10),
+    "lion_bf16_plain": ("Lion", dict(LION, kahan_sum=False), "bfloat16", "group", 10),
+    "lion_bf16_kahan_declr": ("Lion", dict(LION, weight_decay=1e-2, decouple_lr=True, max_lr=3e-4), "bfloat16", "group", 10),
+    "stableadamw_fp32": ("StableAdamW", dict(SADAMW), "float32", "group", 10),
+    "stableadamw_bf16_kahan": ("StableAdamW", dict(SADAMW), "bfloat16", "group", 10),
+    "stableadamw_bf16_plain": ("StableAdamW", dict(SADAMW, kahan_sum=False), "bfloat16", "group", 10),
+    "stableadamw_bf16_kahan_declr": ("StableAdamW", dict(SADAMW, weight_decay=1e-3, decouple_lr=True, max_lr=2e-3), "bfloat16", "group", 10),
+    "adan_fp32": ("Adan", dict(ADAN), "float32", "group", 10),
+    "adan_bf16_kahan": ("Adan", dict(ADAN, kahan_sum=True), "bfloat16", "group", 10),
+    "adan_bf16_plain": ("Adan", dict(ADAN), "bfloat16", "group", 10),
+    "adan_bf16_kahan_declr": ("Adan", dict(ADAN, kahan_sum=True, decouple_lr=True, weight_decay=1e-3), "bfloat16", "group", 10),
+    "adamw_fp32_release": ("AdamW", dict(ADAMW), "float32", "release", 8),
+    "adamw_bf16_kahan_release": ("AdamW", dict(ADAMW), "bfloat16", "release", 8),
+    "lion_bf16_kahan_release": ("Lion", dict(LION), "bfloat16", "release", 8),
+    "stableadamw_bf16_kahan_release": ("StableAdamW", dict(SADAMW), "bfloat16", "release", 8),
+    "adan_bf16_kahan_release": ("Adan", dict(ADAN, kahan_sum=True), "bfloat16", "release", 8),
+}
+
+STATE_KEYS = ("exp_avg", "exp_avg_sq", "exp_avg_diff", "prev_grad", "kahan_comp")
+
+
+def to_np(t: torch.Tensor) -> np.ndarray:
+    t = t.detach().cpu().contiguous()
+    if t.dtype == torch.bfloat16:
+        return t.view(torch.int16).numpy().view(np.uint16).copy()
+    return t.numpy().copy()
+
+
+def grad_scale(step: int) -> float:
+    """Gradient std per step.  Varies so StableAdamW's RMS clip is above 1 on some steps."""
+    return 1e-3 * (1.0, 1.0, 4.0, 0.5, 2.0)[step % 5]
+
+
+def make_inputs(dtype: torch.dtype, n_steps: int, seed: int):
+    gen = torch.Generator().manual_seed(seed)
+    params, grads = [], []
+    for shape in SHAPES:
+        p = torch.randn(shape, generator=gen) * 0.02
+        p.view(-1)[:2] = torch.tensor([0.0, 1.0])
+        params.append(p.to(dtype))
+    for t in range(n_steps):
+        gs = []
+        for shape in SHAPES:
+            g = torch.randn(shape, generator=gen) * grad_scale(t)
+            # special values: zero, below eps, large, and a sign flip partner
+            g.view(-1)[:6] = torch.tensor([0.0, 1e-9, -1e-9, 1.0, -0.5, 3e-7])
+            gs.append(g.to(dtype))
+        grads.append(gs)
+    return params, grads
+
+
+def snapshot(out: dict, tag: str, params, opt):
+    for i, p in enumerate(params):
+        out[f"{tag}.param.{i}"] = to_np(p)
+        st = opt.state[p]
+        for key in STATE_KEYS:
+            if key in st and torch.is_tensor(st[key]) and st[key].numel() == p.numel():
+                out[f"{tag}.{key}.{i}"] = to_np(st[key])
+
+
+def run_case(optimi, name: str, seed: int) -> dict:
+    cls_name, kwargs, dtype_name, mode, n_steps = CASES[name]
+    dtype = getattr(torch, dtype_name)
+    p0, grads = make_inputs(dtype, n_steps, seed)
+    out = {}
+    for i, p in enumerate(p0):
+        out[f"in.param.{i}"] = to_np(p)
+    for t, gs in enumerate(grads):
+        for i, g in enumerate(gs):
+            out[f"in.grad.{t}.{i}"] = to_np(g)
+
+    params = [torch.nn.Parameter(p.clone()) for p in p0]
+    release = mode == "release"
+    opt = getattr(optimi, cls_name)(params, triton=False, foreach=False, gradient_release=release, **kwargs)
+    for t in range(n_steps):
+        if release:
+            opt.optimizer_accumulation = (t + 1) % 4 != 0
+            for i in reversed(range(len(params))):
+                params[i].grad = grads[t][i].clone()
+                opt.step(param=params[i])
+                opt.zero_grad(param=params[i])
+        else:
+            for p, g in zip(params, grads[t]):
+                p.grad = g.clone()
+            opt.step()
+            opt.zero_grad()
+        if (t + 1) in SNAP_STEPS or t + 1 == n_steps:
+            snapshot(out, f"out.{t + 1}", params, opt)
+    return out
+
+
+def main():
+    ref = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+    sys.path.insert(0, ref)
+    import optimi  # noqa: E402  (the reference; CPU for-loop path only)
+
+    torch.set_num_threads(1)
+    for seed, name in enumerate(sorted(CASES)):
+        out = run_case(optimi, name, 1000 + seed)
+        path = os.path.join(HERE, f"{name}.npz")
+        np.savez_compressed(path, **out)
+        print(f"{name}: {len(out)} arrays, {os.path.getsize(path) / 1024:.1f} KiB")
+
+
+if __name__ == "__main__":
+    main()

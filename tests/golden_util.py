@@ -1,0 +1,102 @@
+"""Loading and replaying the golden fixtures (tests/golden/*.npz).
+
+A fixture holds the inputs the reference saw (initial params, the gradient of
+every step) and what its for-loop path produced (params and states after
+selected steps).  ``replay`` feeds the same inputs to any engine with the
+small ``step`` / ``step_param`` interface of ``oracle.forloop.ForLoopRun`` and
+returns the snapshots in the fixture's own key layout.
+"""
+
+from __future__ import annotations
+
+import glob
+import importlib.util
+import os
+
+import numpy as np
+import torch
+
+GOLDEN_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+_spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(GOLDEN_DIR, "make_fixtures.py"))
+_mk = importlib.util.module_from_spec(_spec)
+_spec.loader.exec_module(_mk)
+CASES = _mk.CASES
+STATE_KEYS = _mk.STATE_KEYS
+N_TENSORS = len(_mk.SHAPES)
+
+OPT_NAME = {"Adam": "adam", "AdamW": "adamw", "Lion": "lion", "StableAdamW": "stableadamw", "Adan": "adan"}
+
+
+def case_names():
+    names = sorted(CASES)
+    have = {os.path.basename(p)[:-4] for p in glob.glob(os.path.join(GOLDEN_DIR, "*.npz"))}
+    assert set(names) <= have, f"fixtures missing: {sorted(set(names) - have)}"
+    return names
+
+
+def from_np(a: np.ndarray) -> torch.Tensor:
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+    return torch.from_numpy(a.copy())
+
+
+def load(name: str) -> dict[str, torch.Tensor]:
+    with np.load(os.path.join(GOLDEN_DIR, f"{name}.npz"), allow_pickle=False) as z:
+        return {k: from_np(z[k]) for k in z.files}
+
+
+def snap_steps(fx: dict) -> list[int]:
+    return sorted({int(k.split(".")[1]) for k in fx if k.startswith("out.")})
+
+
+def replay(name: str, fx: dict, make_engine, device="cpu") -> dict[str, torch.Tensor]:
+    """``make_engine(opt_name, params, gradient_release=..., **kwargs)`` → engine."""
+    cls_name, kwargs, _dtype, mode, n_steps = CASES[name]
+    params = [fx[f"in.param.{i}"].clone().to(device) for i in range(N_TENSORS)]
+    release = mode == "release"
+    eng = make_engine(OPT_NAME[cls_name], params, gradient_release=release, **kwargs)
+    wanted = set(snap_steps(fx))
+    out = {}
+    for t in range(n_steps):
+        grads = [fx[f"in.grad.{t}.{i}"].clone().to(device) for i in range(N_TENSORS)]
+        if release:
+            eng.optimizer_accumulation = (t + 1) % 4 != 0
+            for i in reversed(range(N_TENSORS)):
+                eng.step_param(i, grads[i])
+        else:
+            eng.step(grads)
+        if (t + 1) in wanted:
+            for i in range(N_TENSORS):
+                out[f"out.{t + 1}.param.{i}"] = eng.params[i].detach().cpu().clone()
+                for key in STATE_KEYS:
+                    st = eng.state[i].get(key) if eng.state[i] is not None else None
+                    if torch.is_tensor(st) and st.numel() == eng.params[i].numel():
+                        out[f"out.{t + 1}.{key}.{i}"] = st.detach().cpu().clone()
+    return out
+
+
+# ----------------------------------------------------------------------------
+# comparison helpers
+# ----------------------------------------------------------------------------
+def bf16_ordinal(t: torch.Tensor) -> torch.Tensor:
+    """Maps bf16 values to integers so that adjacent representable values differ by 1."""
+    bits = t.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
+    neg = bits >= 0x8000
+    return torch.where(neg, 0x8000 - bits, bits)
+
+
+def bf16_ulp_diff(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    return (bf16_ordinal(a) - bf16_ordinal(b)).abs()
+
+
+def bf16_ulp_of(t: torch.Tensor) -> torch.Tensor:
+    """Size of one bf16 ulp at each value of ``t`` (as fp32)."""
+    f = t.float().abs().clamp_min(2.0**-126)
+    return torch.exp2(torch.floor(torch.log2(f)) - 7)
+
+
+def fp32_rel_err(a: torch.Tensor, b: torch.Tensor, floor: float) -> torch.Tensor:
+    """|a-b| / max(|a|,|b|, floor)."""
+    a, b = a.double(), b.double()
+    return (a - b).abs() / torch.maximum(torch.maximum(a.abs(), b.abs()), torch.tensor(floor, dtype=torch.float64))
