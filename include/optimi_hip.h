@@ -1,0 +1,161 @@
+/*
+ * optimi_hip.h — C ABI of the MI355X (gfx950) fused optimizer-step library.
+ *
+ * The reference (warner-benjamin/optimi) has no FFI: its accelerated backend is a set
+ * of Triton kernels launched from Python, one launch per tensor.  Each entry point
+ * below takes the place of one of those launchers and keeps its argument meaning:
+ * pointers to the parameter, gradient and state buffers, the element count, and the
+ * step scalars already formed by the functional dispatcher (debiased betas, the
+ * weight-decay factor).  Scalars arrive as doubles, exactly as the Python floats the
+ * reference passes, and are narrowed inside the library the way the reference's
+ * PyTorch for-loop path narrows them, because that path defines the results.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a negative optimi_status for a rejected
+ *     argument, or a positive hipError_t value for a HIP runtime failure;
+ *     optimi_hip_error_string() explains either.  Nothing throws.
+ *   - all buffers are device memory of the current HIP device, contiguous, and of
+ *     the one dtype named by `dtype`.  The gradient is never written.
+ *   - work is enqueued on `stream` (a hipStream_t; NULL = the default stream) and
+ *     the call returns without waiting for it.
+ *   - `kahan_comp` may be NULL whenever the Kahan branch is not taken (fp32 tensors,
+ *     OPTIMI_KAHAN unset, or OPTIMI_UPDATE unset).
+ *   - buffers aligned to 16 bytes take the vectorised path; any other alignment is
+ *     accepted and runs an element-wise path.
+ */
+#ifndef OPTIMI_HIP_H
+#define OPTIMI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* optimi_stream_t; /* hipStream_t */
+
+enum optimi_dtype { OPTIMI_F32 = 0, OPTIMI_BF16 = 1 };
+
+enum optimi_flags {
+  OPTIMI_KAHAN = 1,       /* kahan_sum: only acts on bf16 tensors (optimi/adam.py:384)            */
+  OPTIMI_UPDATE = 2,      /* update_parameters; unset = accumulate-only step (optimi/adam.py:308) */
+  OPTIMI_DECOUPLE_WD = 4, /* Adam: decoupled decay p*=factor; unset = L2 (optimi/adam.py:373-377) */
+  OPTIMI_ADAM_WD = 8,     /* Adan: Adam-style decay before the step (optimi/adan.py:447-448)      */
+  OPTIMI_DECOUPLE_LR = 16 /* StableAdamW: fully decoupled decay (optimi/stableadamw.py:453-457)   */
+};
+
+enum optimi_status {
+  OPTIMI_OK = 0,
+  OPTIMI_ERR_NULL = -1,      /* a required pointer is NULL                         */
+  OPTIMI_ERR_SIZE = -2,      /* negative element or tensor count                   */
+  OPTIMI_ERR_DTYPE = -3,     /* dtype is not an optimi_dtype                       */
+  OPTIMI_ERR_ALIGN = -4,     /* a buffer is not aligned to its element size        */
+  OPTIMI_ERR_DEVICE = -5,    /* group used on a device other than the one it was made on */
+  OPTIMI_ERR_NOMEM = -6,     /* host allocation failed                             */
+  OPTIMI_ERR_ARG = -7        /* inconsistent scalar argument (e.g. max_lr <= 0 with OPTIMI_DECOUPLE_LR) */
+};
+
+/* Text for a status returned by any function of this header. */
+const char* optimi_hip_error_string(int status);
+
+/* ABI version of the loaded library (major * 1000 + minor). */
+int optimi_hip_version(void);
+
+/* Elements one workgroup covers for `dtype`; tensors are cut into chunks of this size. */
+int64_t optimi_hip_chunk_elems(int dtype);
+
+/* ---------------------------------------------------------------------------------
+ * Group handle.  Owns what a whole-list launch needs besides the caller's tensors:
+ * the device-side tensor table (pointers, sizes), the chunk map, StableAdamW's
+ * reduction partials and per-tensor scalars, and a small pinned staging ring.  None
+ * of it is optimizer state; it can be dropped and rebuilt at any time.  Tables are
+ * re-uploaded only when a pointer or size differs from the previous call.  A group
+ * belongs to the device that was current when it was created and must be used by
+ * one thread and one stream at a time.  (No counterpart in the reference: it plays
+ * the role of the Python loop in optimi/adam.py:551-583.)
+ * ------------------------------------------------------------------------------- */
+typedef struct optimi_group optimi_group;
+int optimi_hip_group_create(optimi_group** out);
+int optimi_hip_group_destroy(optimi_group* group);
+
+/* ---------------------------------------------------------------------------------
+ * Whole-list steps: one launch covers every tensor of the list.
+ * Arrays of `n_tensors` host pointers to device buffers; numel[i] elements each.
+ * ------------------------------------------------------------------------------- */
+
+/* Adam / AdamW over a list.  Replaces _triton_adam (optimi/adam.py:533-583); results
+ * follow _single_param_adam (optimi/adam.py:354-396).  weight_decay is the formed
+ * factor 1-lr*wd when OPTIMI_DECOUPLE_WD is set, the raw coefficient otherwise, 0 = none. */
+int optimi_hip_adam_multi(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                          void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                          const int64_t* numel, int dtype, double lr, double beta1_comp, double beta2_hat,
+                          double beta2_comp, double weight_decay, double eps, uint32_t flags,
+                          optimi_stream_t stream);
+
+/* Lion over a list.  Replaces _triton_lion (optimi/lion.py:453-492); results follow
+ * _single_param_lion (optimi/lion.py:301-338).  weight_decay is the formed factor, 0 = none. */
+int optimi_hip_lion_multi(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                          void* const* exp_avg, void* const* kahan_comp, const int64_t* numel, int dtype, double lr,
+                          double beta1_comp, double beta2_comp, double weight_decay, uint32_t flags,
+                          optimi_stream_t stream);
+
+/* StableAdamW over a list.  Replaces _triton_stableadamw (optimi/stableadamw.py:657-725);
+ * results follow _single_param_stableadamw (optimi/stableadamw.py:421-472).  Three launches:
+ * moments + per-chunk partial sums of g^2/max(v,eps^2); one workgroup per tensor that turns
+ * the partials into that tensor's clipped lr and decay factor on the device; the update.
+ * weight_decay is the raw coefficient; max_lr is read only with OPTIMI_DECOUPLE_LR. */
+int optimi_hip_stableadamw_multi(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                                 void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                                 const int64_t* numel, int dtype, double lr, double beta1_comp, double beta2_hat,
+                                 double beta2_comp, double weight_decay, double eps, double max_lr, uint32_t flags,
+                                 optimi_stream_t stream);
+
+/* Adan over a list.  Replaces _triton_adan (optimi/adan.py:652-711); results follow
+ * _single_param_adan (optimi/adan.py:405-469).  prev_grad holds the negated previous
+ * gradient.  weight_decay is the formed factor 1+lr*wd (or 1-lr*wd with OPTIMI_ADAM_WD), 0 = none. */
+int optimi_hip_adan_multi(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                          void* const* exp_avg, void* const* exp_avg_diff, void* const* exp_avg_sq,
+                          void* const* prev_grad, void* const* kahan_comp, const int64_t* numel, int dtype, double lr,
+                          double beta1_comp, double beta2, double beta2_comp, double beta3_hat, double beta3_comp,
+                          double eps, double weight_decay, uint32_t flags, optimi_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
+ * Per-tensor steps for gradient release: pointers travel as kernel arguments, no table.
+ * ------------------------------------------------------------------------------- */
+
+/* Replaces _single_param_triton_adam (optimi/adam.py:585-630). */
+int optimi_hip_adam_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* kahan_comp,
+                           int64_t numel, int dtype, double lr, double beta1_comp, double beta2_hat,
+                           double beta2_comp, double weight_decay, double eps, uint32_t flags, optimi_stream_t stream);
+
+/* Replaces _single_param_triton_lion (optimi/lion.py:494-530). */
+int optimi_hip_lion_single(void* param, const void* grad, void* exp_avg, void* kahan_comp, int64_t numel, int dtype,
+                           double lr, double beta1_comp, double beta2_comp, double weight_decay, uint32_t flags,
+                           optimi_stream_t stream);
+
+/* Replaces _single_param_triton_stableadamw (optimi/stableadamw.py:727-791).  `group`
+ * supplies the reduction workspace (the reference keeps a one-float `mean_square` tensor
+ * in the optimizer state for this, optimi/stableadamw.py:129-130). */
+int optimi_hip_stableadamw_single(optimi_group* group, void* param, const void* grad, void* exp_avg, void* exp_avg_sq,
+                                  void* kahan_comp, int64_t numel, int dtype, double lr, double beta1_comp,
+                                  double beta2_hat, double beta2_comp, double weight_decay, double eps, double max_lr,
+                                  uint32_t flags, optimi_stream_t stream);
+
+/* Replaces _single_param_triton_adan (optimi/adan.py:713-770). */
+int optimi_hip_adan_single(void* param, const void* grad, void* exp_avg, void* exp_avg_diff, void* exp_avg_sq,
+                           void* prev_grad, void* kahan_comp, int64_t numel, int dtype, double lr, double beta1_comp,
+                           double beta2, double beta2_comp, double beta3_hat, double beta3_comp, double eps,
+                           double weight_decay, uint32_t flags, optimi_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
+ * Measurement aid (no counterpart in the reference): a plain 16-byte-per-lane copy of
+ * `bytes` bytes (a multiple of 16, both pointers 16-byte aligned).  Benchmarks use it as
+ * the practical bandwidth ceiling and to scale hardware byte counters.
+ * ------------------------------------------------------------------------------- */
+int optimi_hip_copy_probe(void* dst, const void* src, int64_t bytes, optimi_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OPTIMI_HIP_H */

@@ -1,0 +1,18 @@
+"""optimi_amd: the fused optimizer step of optimi, hand-written for MI355X (gfx950).
+
+Drop-in for the accelerated path of warner-benjamin/optimi: the same optimizer classes,
+functional forms, gradient-release hooks and ``state_dict`` layout, with ``triton=True``
+served by HIP kernels behind a C ABI (``include/optimi_hip.h``).
+"""
+
+__version__ = "0.1.0"
+
+from .functional import adam, adamw, adan, lion, stableadamw
+from .gradient_release import prepare_for_gradient_release, remove_gradient_release
+from .optimizers import Adam, AdamW, Adan, Lion, OptimiOptimizer, StableAdamW
+
+__all__ = [
+    "Adam", "AdamW", "Adan", "Lion", "StableAdamW", "OptimiOptimizer",
+    "adam", "adamw", "adan", "lion", "stableadamw",
+    "prepare_for_gradient_release", "remove_gradient_release",
+]

@@ -1,0 +1,80 @@
+"""In-tree build of the two native pieces.
+
+* ``liboptimi_hip.so`` – the gfx950 kernels and the C ABI (hipcc, no torch).
+* ``_C.*.so``          – the PyTorch-ROCm binding over that ABI (g++, host code only).
+
+Both land next to this file so they travel with the source tree.  Run
+``python -m optimi_amd.build`` to build them by hand.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+import sysconfig
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+INCLUDE = os.path.join(ROOT, "include")
+CSRC = os.path.join(HERE, "csrc")
+LIB_PATH = os.path.join(HERE, "liboptimi_hip.so")
+EXT_SUFFIX = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+BINDING_PATH = os.path.join(HERE, "_C" + EXT_SUFFIX)
+ROCM_HOME = os.environ.get("ROCM_HOME", "/opt/rocm")
+
+# -ffp-contract=off: the kernels spell out every fused multiply-add they want.
+# packed-fp32-ops is switched off: hipcc must not form v_pk_*_f32 from the float code.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _run(cmd: list[str]):
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"build step failed ({proc.returncode}): {' '.join(cmd)}\n{proc.stdout}\n{proc.stderr}")
+    return proc
+
+
+def build_lib(verbose: bool = False) -> str:
+    hipcc = shutil.which("hipcc") or os.path.join(ROCM_HOME, "bin", "hipcc")
+    cmd = [hipcc, *HIPCC_FLAGS, f"-I{INCLUDE}", "-o", LIB_PATH, os.path.join(CSRC, "optimi_hip.hip")]
+    if verbose:
+        print(" ".join(cmd))
+    _run(cmd)
+    return LIB_PATH
+
+
+def build_binding(verbose: bool = False) -> str:
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    inc = [f"-I{p}" for p in ce.include_paths()] + [f"-I{INCLUDE}", f"-I{ROCM_HOME}/include",
+                                                     f"-I{sysconfig.get_paths()['include']}"]
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    cmd = [
+        shutil.which("g++") or "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-deprecated-declarations",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H",
+        f"-D_GLIBCXX_USE_CXX11_ABI={abi}", *inc, os.path.join(CSRC, "torch_binding.cpp"), "-o", BINDING_PATH,
+        f"-L{HERE}", "-loptimi_hip", f"-L{torch_lib}", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip",
+        "-ltorch_python", f"-L{ROCM_HOME}/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}",
+        f"-Wl,-rpath,{ROCM_HOME}/lib",
+    ]
+    if verbose:
+        print(" ".join(cmd))
+    _run(cmd)
+    return BINDING_PATH
+
+
+def build_all(verbose: bool = False):
+    build_lib(verbose)
+    build_binding(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    print("built", LIB_PATH, BINDING_PATH, file=sys.stderr)

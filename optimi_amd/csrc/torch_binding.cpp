@@ -1,0 +1,279 @@
+// Thin PyTorch-ROCm binding over the C ABI in optimi_hip.h.
+//
+// PyTorch owns every buffer and the stream; this file only turns tensors into raw
+// pointers, checks that they are what the kernels assume (same device, one supported
+// dtype, equal sizes, the parameter's dense layout), picks the calling thread's current
+// HIP stream and raises RuntimeError when the library returns a non-zero status.  It
+// stands where the reference enters its Triton launchers (optimi/adam.py:278-291,
+// lion.py:240-253, stableadamw.py:337-350, adan.py:314-327).
+
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include <cmath>
+#include <optional>
+#include <vector>
+
+#include "optimi_hip.h"
+
+namespace {
+
+using TensorList = std::vector<at::Tensor>;
+using OptTensorList = std::vector<std::optional<at::Tensor>>;
+
+void check_status(int rc, const char* what) {
+  TORCH_CHECK(rc == 0, what, " failed: ", optimi_hip_error_string(rc), " (status ", rc, ")");
+}
+
+int dtype_code(const at::Tensor& t) {
+  switch (t.scalar_type()) {
+    case at::kFloat: return OPTIMI_F32;
+    case at::kBFloat16: return OPTIMI_BF16;
+    default: TORCH_CHECK(false, "optimi_amd: unsupported parameter dtype ", t.scalar_type(), " (float32 and bfloat16 are implemented)");
+  }
+  return -1;
+}
+
+// A buffer may stand in for the parameter element by element only when it has the
+// parameter's dtype, device, size and strides.
+void check_like(const at::Tensor& ref, const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.device() == ref.device(), "optimi_amd: ", name, " is on ", t.device(), ", parameter on ", ref.device());
+  TORCH_CHECK(t.scalar_type() == ref.scalar_type(), "optimi_amd: ", name, " has dtype ", t.scalar_type(), ", parameter ", ref.scalar_type());
+  TORCH_CHECK(t.numel() == ref.numel(), "optimi_amd: ", name, " has ", t.numel(), " elements, parameter ", ref.numel());
+  TORCH_CHECK(t.strides() == ref.strides(), "optimi_amd: ", name, " strides differ from the parameter's");
+}
+
+void check_param(const at::Tensor& p) {
+  TORCH_CHECK(p.is_cuda(), "optimi_amd: parameters must live on a HIP device, got ", p.device());
+  TORCH_CHECK(p.is_non_overlapping_and_dense(), "optimi_amd: parameter must be dense and non-overlapping in memory");
+}
+
+class Group {
+ public:
+  Group() { check_status(optimi_hip_group_create(&g_), "optimi_hip_group_create"); }
+  ~Group() {
+    if (g_) (void)optimi_hip_group_destroy(g_);
+  }
+  Group(const Group&) = delete;
+  Group& operator=(const Group&) = delete;
+  optimi_group* get() const { return g_; }
+
+ private:
+  optimi_group* g_ = nullptr;
+};
+
+// Collects the raw pointers of a list that must match `params` tensor by tensor.
+struct PtrList {
+  std::vector<void*> v;
+  void* const* data() const { return v.data(); }
+  const void* const* cdata() const { return (const void* const*)v.data(); }
+};
+
+PtrList gather(const TensorList& params, const TensorList& list, const char* name) {
+  TORCH_CHECK(list.size() == params.size(), "optimi_amd: ", name, " has ", list.size(), " tensors, params has ", params.size());
+  PtrList out;
+  out.v.reserve(list.size());
+  for (size_t i = 0; i < list.size(); ++i) {
+    check_like(params[i], list[i], name);
+    out.v.push_back(list[i].data_ptr());
+  }
+  return out;
+}
+
+// Kahan buffers: taken only when the Kahan branch runs; placeholders and None are ignored.
+PtrList gather_kahan(const TensorList& params, const OptTensorList& list, bool needed) {
+  PtrList out;
+  if (!needed) return out;
+  TORCH_CHECK(list.size() == params.size(), "optimi_amd: kahan_comps has ", list.size(), " tensors, params has ", params.size());
+  out.v.reserve(list.size());
+  for (size_t i = 0; i < list.size(); ++i) {
+    TORCH_CHECK(list[i].has_value(), "optimi_amd: kahan_sum is on but a Kahan buffer is missing");
+    check_like(params[i], *list[i], "kahan_comp");
+    out.v.push_back(list[i]->data_ptr());
+  }
+  return out;
+}
+
+struct Prepared {
+  int dtype = OPTIMI_F32;
+  bool kahan = false;
+  std::vector<int64_t> numel;
+  PtrList params;
+};
+
+Prepared prepare(const TensorList& params, uint32_t flags) {
+  Prepared pr;
+  if (params.empty()) return pr;
+  pr.dtype = dtype_code(params[0]);
+  pr.kahan = pr.dtype == OPTIMI_BF16 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
+  pr.numel.reserve(params.size());
+  pr.params.v.reserve(params.size());
+  for (const at::Tensor& p : params) {
+    check_param(p);
+    TORCH_CHECK(p.device() == params[0].device(), "optimi_amd: one launch covers one device");
+    TORCH_CHECK(p.scalar_type() == params[0].scalar_type(), "optimi_amd: one launch covers one dtype");
+    pr.numel.push_back(p.numel());
+    pr.params.v.push_back(p.data_ptr());
+  }
+  return pr;
+}
+
+void adam_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
+                const TensorList& exp_avg_sqs, const OptTensorList& kahan_comps, double lr, double beta1_comp,
+                double beta2_hat, double beta2_comp, double weight_decay, double eps, uint32_t flags) {
+  if (params.empty()) return;
+  Prepared pr = prepare(params, flags);
+  PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
+  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  c10::hip::HIPGuard guard(params[0].device());
+  check_status(optimi_hip_adam_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
+                                     pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp, beta2_hat,
+                                     beta2_comp, weight_decay, eps, flags, c10::hip::getCurrentHIPStream().stream()),
+               "optimi_hip_adam_multi");
+}
+
+void lion_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
+                const OptTensorList& kahan_comps, double lr, double beta1_comp, double beta2_comp, double weight_decay,
+                uint32_t flags) {
+  if (params.empty()) return;
+  Prepared pr = prepare(params, flags);
+  PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg");
+  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  c10::hip::HIPGuard guard(params[0].device());
+  check_status(optimi_hip_lion_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(),
+                                     pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp, beta2_comp,
+                                     weight_decay, flags, c10::hip::getCurrentHIPStream().stream()),
+               "optimi_hip_lion_multi");
+}
+
+void stableadamw_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
+                       const TensorList& exp_avg_sqs, const OptTensorList& kahan_comps, double lr, double beta1_comp,
+                       double beta2_hat, double beta2_comp, double weight_decay, double eps, double max_lr,
+                       uint32_t flags) {
+  if (params.empty()) return;
+  Prepared pr = prepare(params, flags);
+  PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
+  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  c10::hip::HIPGuard guard(params[0].device());
+  check_status(optimi_hip_stableadamw_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
+                                            pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp,
+                                            beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags,
+                                            c10::hip::getCurrentHIPStream().stream()),
+               "optimi_hip_stableadamw_multi");
+}
+
+void adan_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
+                const TensorList& exp_avg_diffs, const TensorList& exp_avg_sqs, const TensorList& prev_grads,
+                const OptTensorList& kahan_comps, double lr, double beta1_comp, double beta2, double beta2_comp,
+                double beta3_hat, double beta3_comp, double eps, double weight_decay, uint32_t flags) {
+  if (params.empty()) return;
+  Prepared pr = prepare(params, flags);
+  PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg");
+  PtrList df = gather(params, exp_avg_diffs, "exp_avg_diff"), n = gather(params, exp_avg_sqs, "exp_avg_sq");
+  PtrList pg = gather(params, prev_grads, "prev_grad");
+  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  c10::hip::HIPGuard guard(params[0].device());
+  check_status(optimi_hip_adan_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), df.data(),
+                                     n.data(), pg.data(), pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr,
+                                     beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay, flags,
+                                     c10::hip::getCurrentHIPStream().stream()),
+               "optimi_hip_adan_multi");
+}
+
+// ---- per-tensor entry points (gradient release) --------------------------------------
+struct One {
+  int dtype;
+  bool kahan;
+  void* k = nullptr;
+};
+
+One prepare_one(const at::Tensor& p, const std::optional<at::Tensor>& kahan_comp, uint32_t flags) {
+  check_param(p);
+  One o;
+  o.dtype = dtype_code(p);
+  o.kahan = o.dtype == OPTIMI_BF16 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
+  if (o.kahan) {
+    TORCH_CHECK(kahan_comp.has_value(), "optimi_amd: kahan_sum is on but the Kahan buffer is missing");
+    check_like(p, *kahan_comp, "kahan_comp");
+    o.k = kahan_comp->data_ptr();
+  }
+  return o;
+}
+
+void adam_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
+                 const std::optional<at::Tensor>& kahan_comp, double lr, double beta1_comp, double beta2_hat,
+                 double beta2_comp, double weight_decay, double eps, uint32_t flags) {
+  One o = prepare_one(p, kahan_comp, flags);
+  check_like(p, g, "grad");
+  check_like(p, m, "exp_avg");
+  check_like(p, v, "exp_avg_sq");
+  c10::hip::HIPGuard guard(p.device());
+  check_status(optimi_hip_adam_single(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), o.k, p.numel(), o.dtype, lr,
+                                      beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, flags,
+                                      c10::hip::getCurrentHIPStream().stream()),
+               "optimi_hip_adam_single");
+}
+
+void lion_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const std::optional<at::Tensor>& kahan_comp,
+                 double lr, double beta1_comp, double beta2_comp, double weight_decay, uint32_t flags) {
+  One o = prepare_one(p, kahan_comp, flags);
+  check_like(p, g, "grad");
+  check_like(p, m, "exp_avg");
+  c10::hip::HIPGuard guard(p.device());
+  check_status(optimi_hip_lion_single(p.data_ptr(), g.data_ptr(), m.data_ptr(), o.k, p.numel(), o.dtype, lr, beta1_comp,
+                                      beta2_comp, weight_decay, flags, c10::hip::getCurrentHIPStream().stream()),
+               "optimi_hip_lion_single");
+}
+
+void stableadamw_single(Group& group, const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
+                        const std::optional<at::Tensor>& kahan_comp, double lr, double beta1_comp, double beta2_hat,
+                        double beta2_comp, double weight_decay, double eps, double max_lr, uint32_t flags) {
+  One o = prepare_one(p, kahan_comp, flags);
+  check_like(p, g, "grad");
+  check_like(p, m, "exp_avg");
+  check_like(p, v, "exp_avg_sq");
+  c10::hip::HIPGuard guard(p.device());
+  check_status(optimi_hip_stableadamw_single(group.get(), p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), o.k,
+                                             p.numel(), o.dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps,
+                                             max_lr, flags, c10::hip::getCurrentHIPStream().stream()),
+               "optimi_hip_stableadamw_single");
+}
+
+void adan_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& df, const at::Tensor& n,
+                 const at::Tensor& pg, const std::optional<at::Tensor>& kahan_comp, double lr, double beta1_comp,
+                 double beta2, double beta2_comp, double beta3_hat, double beta3_comp, double eps, double weight_decay,
+                 uint32_t flags) {
+  One o = prepare_one(p, kahan_comp, flags);
+  check_like(p, g, "grad");
+  check_like(p, m, "exp_avg");
+  check_like(p, df, "exp_avg_diff");
+  check_like(p, n, "exp_avg_sq");
+  check_like(p, pg, "prev_grad");
+  c10::hip::HIPGuard guard(p.device());
+  check_status(optimi_hip_adan_single(p.data_ptr(), g.data_ptr(), m.data_ptr(), df.data_ptr(), n.data_ptr(), pg.data_ptr(),
+                                      o.k, p.numel(), o.dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp,
+                                      eps, weight_decay, flags, c10::hip::getCurrentHIPStream().stream()),
+               "optimi_hip_adan_single");
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
+  mod.doc() = "PyTorch-ROCm binding of the optimi_hip C ABI";
+  mod.attr("KAHAN") = (uint32_t)OPTIMI_KAHAN;
+  mod.attr("UPDATE") = (uint32_t)OPTIMI_UPDATE;
+  mod.attr("DECOUPLE_WD") = (uint32_t)OPTIMI_DECOUPLE_WD;
+  mod.attr("ADAM_WD") = (uint32_t)OPTIMI_ADAM_WD;
+  mod.attr("DECOUPLE_LR") = (uint32_t)OPTIMI_DECOUPLE_LR;
+  mod.def("abi_version", &optimi_hip_version);
+  py::class_<Group>(mod, "Group").def(py::init<>());
+  mod.def("adam_multi", &adam_multi);
+  mod.def("lion_multi", &lion_multi);
+  mod.def("stableadamw_multi", &stableadamw_multi);
+  mod.def("adan_multi", &adan_multi);
+  mod.def("adam_single", &adam_single);
+  mod.def("lion_single", &lion_single);
+  mod.def("stableadamw_single", &stableadamw_single);
+  mod.def("adan_single", &adan_single);
+}

@@ -1,0 +1,482 @@
+"""Optimizer classes with the reference's constructor signatures and ``state_dict`` layout.
+
+``OptimiOptimizer`` carries what the reference's base class does (optimi/optimizer.py:12-114):
+argument validation, the fully-decoupled weight-decay warning, gradient-release setup, the
+``optimizer_accumulation`` switch, and ``step`` / ``zero_grad`` on one parameter.  The step
+itself is shared: a subclass only declares its hyper-parameters, its state buffers and which
+functional form to call.  Launch workspaces live in ``self._hip_groups``, outside ``state``
+and ``param_groups``, so checkpoints hold exactly the reference's keys.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Callable, Iterable
+from typing import Any
+from warnings import warn
+
+import torch
+from torch import Tensor
+from torch.optim.optimizer import Optimizer
+
+from . import functional as F
+
+__all__ = ["OptimiOptimizer", "Adam", "AdamW", "Lion", "StableAdamW", "Adan"]
+
+_LOW_PRECISION = (torch.float16, torch.bfloat16)
+
+
+def _default_to_fused(params: list[Tensor]) -> bool:
+    """The reference picks its accelerated backend when every parameter is a plain floating
+    tensor on a bf16-capable GPU (optimi/utils.py:193-201); same rule, HIP devices only."""
+    return all(p is None or (type(p) in (Tensor, torch.nn.Parameter) and p.is_cuda and torch.is_floating_point(p))
+               for p in params)
+
+
+def _check_betas(betas):
+    for i, b in enumerate(betas):
+        if not 0.0 <= b < 1.0:
+            raise ValueError(f"Invalid beta{i + 1} parameter: betas[{i}]={b}")
+
+
+class OptimiOptimizer(Optimizer):
+    """Provides common functionality for optimi optimizers."""
+
+    # subclasses fill these in
+    _moment_keys: tuple[str, ...] = ()      # zero-initialised buffers shaped like the parameter
+    _has_step = True                        # Lion keeps no step counter
+    _kahan_placeholder_dtype: torch.dtype | None = torch.uint8  # None: use the parameter dtype (Lion)
+    _setup_before_state = False             # StableAdamW resolves its backend before touching state
+    _step_state_from_group = True           # per-parameter counter keyed on the group's gradient_release flag (Adan: on the call)
+
+    def __init__(self, params: Iterable[Tensor] | Iterable[dict], defaults: dict[str, Any]):
+        if not 0.0 <= defaults["lr"]:
+            raise ValueError(f"Invalid learning rate: lr={defaults['lr']}")
+        if not 0.0 <= defaults["weight_decay"]:
+            raise ValueError(f"Invalid weight decay: weight_decay={defaults['weight_decay']}")
+        if defaults["decouple_lr"] and defaults["max_lr"] is None:
+            defaults["max_lr"] = defaults["lr"]
+        if defaults["max_lr"] is not None and not 0.0 <= defaults["max_lr"]:
+            raise ValueError(f"Invalid maximum learning rate: max_lr={defaults['max_lr']}")
+        if defaults["foreach"]:
+            raise ValueError("optimi_amd has no foreach backend (the reference deprecates it); leave foreach unset")
+        if defaults["triton"] is False:
+            raise ValueError("optimi_amd implements only the fused HIP backend; leave triton unset or pass triton=True")
+
+        super().__init__(params, defaults)
+
+        if self.defaults.get("decouple_lr", False):
+            high = [g["weight_decay"] for g in self.param_groups
+                    if g.get("decouple_lr", False) and g.get("weight_decay", 0.0) >= 1e-3]
+            if high:
+                warn(
+                    f"You are using weight_decay up to {max(high)} which is potentially high for decouple_lr=True"
+                    f". Unlike decoupled weight decay, fully decoupled weight decay does not reduce weight decay by the learning rate.",
+                    category=UserWarning,
+                )
+
+        self._optimizer_accumulation = False
+        self._hip_groups: dict = {}
+
+        if self.defaults["gradient_release"]:
+            self.defaults["foreach"] = False
+            for group in self.param_groups:
+                group["foreach"] = False
+                for p in group["params"]:
+                    self.state[p]["group"] = group
+
+    # -- pickling: launch workspaces are device handles, never part of a checkpoint --------
+    def __getstate__(self):
+        state = super().__getstate__()
+        state = dict(state)
+        state.pop("_hip_groups", None)
+        return state
+
+    def __setstate__(self, state):
+        super().__setstate__(state)
+        self.__dict__.setdefault("_hip_groups", {})
+        self.__dict__.setdefault("_optimizer_accumulation", False)
+
+    @property
+    def optimizer_accumulation(self) -> bool:
+        "Accumulate gradients in optimizer states during gradient release instead of a full step."
+        return self._optimizer_accumulation
+
+    @optimizer_accumulation.setter
+    def optimizer_accumulation(self, optimizer_accumulation: bool):
+        self._optimizer_accumulation = optimizer_accumulation
+
+    # -- state ---------------------------------------------------------------------------
+    def _extra_state(self, group, state, param):
+        """Hook for subclasses: state entries beyond the moment buffers."""
+
+    def _init_state(self, group: dict[str, Any], state: dict, param: Tensor, gradient_release: bool | None = None):
+        if "kahan_comp" in state:
+            return
+        for key in self._moment_keys:
+            state[key] = torch.zeros_like(param, memory_format=torch.preserve_format)
+        self._extra_state(group, state, param)
+        if (group["kahan_sum"] or group["kahan_sum"] is None) and param.dtype in _LOW_PRECISION:
+            state["kahan_comp"] = torch.zeros_like(param, memory_format=torch.preserve_format)
+            group["kahan_sum"] = True
+        elif group["triton"]:
+            state["kahan_comp"] = torch.zeros(1, dtype=self._kahan_placeholder_dtype or param.dtype, device=param.device)
+        else:
+            state["kahan_comp"] = None
+        self._after_kahan_state(group, state, param)
+        release = group["gradient_release"] if self._step_state_from_group else bool(gradient_release)
+        if release and self._has_step:
+            state["step"] = torch.tensor(0, dtype=torch.int32)
+
+    def _after_kahan_state(self, group, state, param):
+        """Hook for subclasses: state entries the reference creates after ``kahan_comp``."""
+
+    def _setup_group(self, group, params):
+        if group["setup"]:
+            return
+        group["setup"] = True
+        if self._has_step:
+            group["step"] = torch.tensor(0, dtype=torch.int32)
+        if group["triton"] is None:
+            group["triton"] = _default_to_fused(params)
+        self._after_setup(group)
+
+    def _after_setup(self, group):
+        """Hook for subclasses."""
+
+    def _collect(self, group):
+        """Parameters of ``group`` that have a gradient, with their states created."""
+        params = []
+        if self._setup_before_state:
+            self._setup_group(group, params)
+        for p in group["params"]:
+            if p.grad is None:
+                continue
+            params.append(p)
+            self._init_state(group, self.state[p], p)
+        if not self._setup_before_state:
+            self._setup_group(group, params)
+        return params
+
+    # -- the step ------------------------------------------------------------------------
+    def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
+        raise NotImplementedError
+
+    @torch.no_grad()
+    def step(self, closure: Callable | None = None, param: Tensor | None = None):
+        """Performs a single optimization step on the whole model or individual parameter.
+
+        Args:
+            closure: A closure which reevaluates the model and returns the loss. Incompatible with
+                performing an optimization step on a single `param`.
+            param: An individual parameter to perform a fused optimization step during the backward
+                pass. Requires optimizer to be initialized with `gradient_release=True` and model
+                hooks created with `prepare_for_gradient_release`. Incompatible with `closure`.
+        """
+        loss = None
+        if closure is not None and param is None:
+            with torch.enable_grad():
+                loss = closure()
+
+        if param is None:
+            for group in self.param_groups:
+                params = self._collect(group)
+                if not params:
+                    continue
+                if not group["triton"]:
+                    raise RuntimeError(
+                        "optimi_amd: this parameter group cannot use the HIP backend (parameters must be plain "
+                        "floating-point tensors on a HIP device) and there is no other backend"
+                    )
+                states = [self.state[p] for p in params]
+                self._functional(group, params, [p.grad for p in params], states, group.get("step"), False, False)
+        else:
+            state = self.state[param]
+            group = state["group"]
+            if group["triton"] is None:
+                group["triton"] = _default_to_fused([param])
+            self._init_state(group, state, param, True)
+            if not group["triton"]:
+                raise RuntimeError("optimi_amd: parameter is not eligible for the HIP backend and there is no other backend")
+            self._functional(group, param, param.grad, state, state.get("step"), True, self._optimizer_accumulation)
+        return loss
+
+    @torch._disable_dynamo
+    def zero_grad(self, set_to_none: bool = True, param: Tensor | None = None):
+        """Resets the gradients of all optimized parameters or individual parameter.
+
+        Args:
+            set_to_none: If True, the gradients will be deallocated after the call (default: True)
+            param: Resets the gradients of the passed `param`. For use with `gradient_release=True`.
+        """
+        if param is None:
+            super().zero_grad(set_to_none=set_to_none)
+        elif param.grad is not None:
+            if set_to_none:
+                param.grad = None
+            elif param.grad.grad_fn is not None:
+                param.grad.detach_()
+            else:
+                param.grad.requires_grad_(False)
+
+
+def _col(states, key):
+    """A state entry for one parameter (dict) or the list of it over many (list of dicts)."""
+    return states[key] if isinstance(states, dict) else [s[key] for s in states]
+
+
+class Adam(OptimiOptimizer):
+    """Adam optimizer. Optionally with decoupled weight decay (AdamW).
+
+    Args:
+        params: Iterable of parameters to optimize or dicts defining parameter groups
+        lr: Learning rate
+        betas: Coefficients for gradient and squared gradient moving averages (default: (0.9, 0.99))
+        weight_decay: Weight decay coefficient. If `decouple_wd` and `decouple_lr` are False,
+            applies L2 penalty (default: 0)
+        eps: Added to denominator to improve numerical stability (default: 1e-6)
+        decouple_wd: Apply decoupled weight decay instead of L2 penalty (default: False)
+        decouple_lr: Apply fully decoupled weight decay instead of L2 penalty (default: False)
+        max_lr: Maximum scheduled learning rate. Set if `lr` is not the maximum scheduled learning
+            rate and `decouple_lr` is True (default: None)
+        kahan_sum: Enables Kahan summation for more accurate parameter updates when training in low
+            precision (bfloat16). If unspecified, automatically applies for low precision
+            parameters (default: None)
+        foreach: Not available in this package; must stay unset (default: None)
+        triton: Selects the fused backend, here the HIP kernels. Unset or True (default: None)
+        gradient_release: Fuses optimizer step and zero_grad as part of the parameter's backward
+            pass. Requires model hooks created with `prepare_for_gradient_release`. Incompatible
+            with closure (default: False)
+    """
+
+    _moment_keys = ("exp_avg", "exp_avg_sq")
+
+    def __init__(
+        self,
+        params: Iterable[Tensor] | Iterable[dict],
+        lr: float,
+        betas: tuple[float, float] = (0.9, 0.99),
+        weight_decay: float = 0,
+        eps: float = 1e-6,
+        decouple_wd: bool = False,
+        decouple_lr: bool = False,
+        max_lr: float | None = None,
+        kahan_sum: bool | None = None,
+        foreach: bool | None = None,
+        triton: bool | None = None,
+        gradient_release: bool = False,
+    ):
+        _check_betas(betas)
+        if not 0.0 <= eps:
+            raise ValueError(f"Invalid epsilon: {eps=}")
+        defaults = dict(lr=lr, beta1=betas[0], beta2=betas[1], eps=eps, weight_decay=weight_decay,
+                        decouple_wd=decouple_wd, decouple_lr=decouple_lr, max_lr=max_lr, kahan_sum=kahan_sum,
+                        foreach=foreach, triton=triton, gradient_release=gradient_release, setup=False)
+        super().__init__(params, defaults)
+
+    def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
+        F.adam(params, grads, _col(states, "exp_avg"), _col(states, "exp_avg_sq"), _col(states, "kahan_comp"),
+               lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"], weight_decay=group["weight_decay"],
+               eps=group["eps"], step=step, decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"],
+               max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=group["triton"],
+               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
+
+
+class AdamW(Adam):
+    """AdamW optimizer: Adam with decoupled weight decay.
+
+    Args as `Adam`, without `decouple_wd` (always on) and with `weight_decay` defaulting to 1e-2.
+    """
+
+    def __init__(
+        self,
+        params: Iterable[Tensor] | Iterable[dict],
+        lr: float,
+        betas: tuple[float, float] = (0.9, 0.99),
+        weight_decay: float = 1e-2,
+        eps: float = 1e-6,
+        decouple_lr: bool = False,
+        max_lr: float | None = None,
+        kahan_sum: bool | None = None,
+        foreach: bool | None = None,
+        triton: bool | None = None,
+        gradient_release: bool = False,
+    ):
+        super().__init__(params=params, lr=lr, betas=betas, weight_decay=weight_decay, eps=eps, decouple_wd=True,
+                         decouple_lr=decouple_lr, max_lr=max_lr, kahan_sum=kahan_sum, foreach=foreach, triton=triton,
+                         gradient_release=gradient_release)
+
+
+class Lion(OptimiOptimizer):
+    """Lion optimizer. Evolved Sign Momentum.
+
+    Args:
+        params: Iterable of parameters to optimize or dicts defining parameter groups
+        lr: Learning rate
+        betas: Coefficients for update moving average and gradient moving average (default: (0.9, 0.99))
+        weight_decay: Weight decay coefficient. If `decouple_lr` is False, applies decoupled
+            weight decay (default: 0)
+        decouple_lr: Apply fully decoupled weight decay instead of decoupled weight decay (default: False)
+        max_lr: Maximum scheduled learning rate. Set if `lr` is not the maximum scheduled learning
+            rate and `decouple_lr` is True (default: None)
+        kahan_sum, foreach, triton, gradient_release: as `Adam`
+    """
+
+    _moment_keys = ("exp_avg",)
+    _has_step = False
+    _kahan_placeholder_dtype = None
+
+    def __init__(
+        self,
+        params: Iterable[Tensor] | Iterable[dict],
+        lr: float,
+        betas: tuple[float, float] = (0.9, 0.99),
+        weight_decay: float = 0,
+        decouple_lr: bool = False,
+        max_lr: float | None = None,
+        kahan_sum: bool | None = None,
+        foreach: bool | None = None,
+        triton: bool | None = None,
+        gradient_release: bool = False,
+    ):
+        _check_betas(betas)
+        defaults = dict(lr=lr, beta1=betas[0], beta2=betas[1], weight_decay=weight_decay, decouple_lr=decouple_lr,
+                        max_lr=max_lr, kahan_sum=kahan_sum, foreach=foreach, triton=triton,
+                        gradient_release=gradient_release, setup=False)
+        super().__init__(params, defaults)
+
+    def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
+        F.lion(params, grads, _col(states, "exp_avg"), _col(states, "kahan_comp"), lr=group["lr"], beta1=group["beta1"],
+               beta2=group["beta2"], weight_decay=group["weight_decay"], decouple_lr=group["decouple_lr"],
+               max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=group["triton"],
+               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
+
+
+def _restore_scratch_state(optim: OptimiOptimizer):
+    """``load_state_dict`` casts floating state to the parameter dtype; bring the fp32 scratch
+    back (optimi/stableadamw.py:38-47)."""
+    for group in optim.param_groups:
+        if group["triton"]:
+            for p in group["params"]:
+                state = optim.state[p]
+                if "mean_square" in state:
+                    state["mean_square"] = state["mean_square"].to(dtype=torch.float32, device=p.device)
+                else:
+                    state["mean_square"] = torch.zeros(1, dtype=torch.float32, device=p.device)
+
+
+class StableAdamW(OptimiOptimizer):
+    """StableAdamW optimizer. An AdamW-Adafactor hybrid with learning rate update clipping.
+
+    Args:
+        params: Iterable of parameters to optimize or dicts defining parameter groups
+        lr: Learning rate
+        betas: Coefficients for gradient and squared gradient moving averages (default: (0.9, 0.99))
+        weight_decay: Weight decay coefficient. If `decouple_lr` is False, applies decoupled weight
+            decay (default: 1e-2)
+        eps: Added to denominator to improve numerical stability (default: 1e-6)
+        decouple_lr, max_lr, kahan_sum, foreach, triton, gradient_release: as `Adam`
+    """
+
+    _moment_keys = ("exp_avg", "exp_avg_sq")
+    _setup_before_state = True
+
+    def __init__(
+        self,
+        params: Iterable[Tensor] | Iterable[dict],
+        lr: float,
+        betas: tuple[float, float] = (0.9, 0.99),
+        weight_decay: float = 1e-2,
+        eps: float = 1e-6,
+        decouple_lr: bool = False,
+        max_lr: float | None = None,
+        kahan_sum: bool | None = None,
+        foreach: bool | None = None,
+        triton: bool | None = None,
+        gradient_release: bool = False,
+    ):
+        _check_betas(betas)
+        if not 0.0 <= eps:
+            raise ValueError(f"Invalid epsilon: {eps=}")
+        defaults = dict(lr=lr, beta1=betas[0], beta2=betas[1], eps=eps, weight_decay=weight_decay,
+                        decouple_lr=decouple_lr, max_lr=max_lr, kahan_sum=kahan_sum, foreach=foreach, triton=triton,
+                        gradient_release=gradient_release, setup=False)
+        super().__init__(params, defaults)
+        self.register_load_state_dict_post_hook(_restore_scratch_state)
+
+    def _extra_state(self, group, state, param):
+        state["eps_sq"] = torch.tensor(group["eps"] ** 2, dtype=param.dtype, device=param.device)
+
+    def _after_kahan_state(self, group, state, param):
+        if group["triton"]:
+            state["mean_square"] = torch.zeros(1, dtype=torch.float32, device=param.device)
+
+    def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
+        F.stableadamw(params, grads, _col(states, "exp_avg"), _col(states, "exp_avg_sq"), _col(states, "eps_sq"),
+                      _col(states, "kahan_comp"), lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"],
+                      weight_decay=group["weight_decay"], eps=group["eps"], step=step, decouple_lr=group["decouple_lr"],
+                      max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=group["triton"],
+                      gradient_release=gradient_release, optimizer_accumulation=accumulate, mean_squares=None,
+                      _groups=self._hip_groups)
+
+
+class Adan(OptimiOptimizer):
+    """Adan Optimizer: Adaptive Nesterov Momentum Algorithm.
+
+    Args:
+        params: Iterable of parameters to optimize or dicts defining parameter groups
+        lr: Learning rate
+        betas: Coefficients for gradient, gradient difference, and squared gradient moving
+            averages (default: (0.98, 0.92, 0.99))
+        weight_decay: Weight decay coefficient. If `decouple_lr` is False, applies decoupled
+            weight decay (default: 2e-2)
+        eps: Added to denominator to improve numerical stability (default: 1e-6)
+        decouple_lr, max_lr: as `Adam`
+        adam_wd: Apply weight decay before parameter update (Adam-style), instead of after the
+            update per Adan algorithm (default: False)
+        kahan_sum: Enables Kahan summation for low precision parameters (default: False)
+        foreach, triton, gradient_release: as `Adam`
+    """
+
+    _moment_keys = ("exp_avg", "exp_avg_diff", "exp_avg_sq")
+    _step_state_from_group = False
+
+    def __init__(
+        self,
+        params: Iterable[Tensor] | Iterable[dict],
+        lr: float,
+        betas: tuple[float, float, float] = (0.98, 0.92, 0.99),
+        weight_decay: float = 2e-2,
+        eps: float = 1e-6,
+        decouple_lr: bool = False,
+        max_lr: float | None = None,
+        adam_wd: bool = False,
+        kahan_sum: bool | None = False,
+        foreach: bool | None = None,
+        triton: bool | None = None,
+        gradient_release: bool = False,
+    ):
+        _check_betas(betas)
+        if not 0.0 <= eps:
+            raise ValueError(f"Invalid epsilon: {eps=}")
+        defaults = dict(lr=lr, beta1=betas[0], beta2=betas[1], beta3=betas[2], eps=eps, weight_decay=weight_decay,
+                        decouple_lr=decouple_lr, max_lr=max_lr, adam_wd=adam_wd, kahan_sum=kahan_sum, foreach=foreach,
+                        triton=triton, gradient_release=gradient_release, setup=False)
+        super().__init__(params, defaults)
+
+    def _extra_state(self, group, state, param):
+        # negated first gradient, so the first difference g_1 - g_0 is zero (optimi/adan.py:109)
+        state["prev_grad"] = param.grad.clone().mul_(-1)
+
+    def _after_setup(self, group):
+        if group["kahan_sum"]:
+            group["adam_wd"] = False
+
+    def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
+        # like the reference class, adam_wd is not forwarded: decay is always Adan-style
+        # (optimi/adan.py:181-203)
+        F.adan(params, grads, _col(states, "exp_avg"), _col(states, "exp_avg_diff"), _col(states, "exp_avg_sq"),
+               _col(states, "prev_grad"), _col(states, "kahan_comp"), lr=group["lr"], beta1=group["beta1"],
+               beta2=group["beta2"], beta3=group["beta3"], eps=group["eps"], weight_decay=group["weight_decay"],
+               step=step, decouple_lr=group["decouple_lr"], max_lr=group["max_lr"], kahan_sum=group["kahan_sum"],
+               foreach=False, triton=group["triton"], gradient_release=gradient_release,
+               optimizer_accumulation=accumulate, _groups=self._hip_groups)
