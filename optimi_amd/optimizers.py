@@ -180,9 +180,7 @@ class OptimiOptimizer(Optimizer):
         if param is None:
             for group in self.param_groups:
                 params = self._collect(group)
-                if not params:
-                    continue
-                if not group["triton"]:
+                if params and not group["triton"]:
                     raise RuntimeError(
                         "optimi_amd: this parameter group cannot use the HIP backend (parameters must be plain "
                         "floating-point tensors on a HIP device) and there is no other backend"
@@ -277,7 +275,7 @@ class Adam(OptimiOptimizer):
         F.adam(params, grads, _col(states, "exp_avg"), _col(states, "exp_avg_sq"), _col(states, "kahan_comp"),
                lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"], weight_decay=group["weight_decay"],
                eps=group["eps"], step=step, decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"],
-               max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=group["triton"],
+               max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
 
@@ -347,7 +345,7 @@ class Lion(OptimiOptimizer):
     def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
         F.lion(params, grads, _col(states, "exp_avg"), _col(states, "kahan_comp"), lr=group["lr"], beta1=group["beta1"],
                beta2=group["beta2"], weight_decay=group["weight_decay"], decouple_lr=group["decouple_lr"],
-               max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=group["triton"],
+               max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
 
@@ -414,7 +412,7 @@ class StableAdamW(OptimiOptimizer):
         F.stableadamw(params, grads, _col(states, "exp_avg"), _col(states, "exp_avg_sq"), _col(states, "eps_sq"),
                       _col(states, "kahan_comp"), lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"],
                       weight_decay=group["weight_decay"], eps=group["eps"], step=step, decouple_lr=group["decouple_lr"],
-                      max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=group["triton"],
+                      max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
                       gradient_release=gradient_release, optimizer_accumulation=accumulate, mean_squares=None,
                       _groups=self._hip_groups)
 
@@ -478,5 +476,5 @@ class Adan(OptimiOptimizer):
                _col(states, "prev_grad"), _col(states, "kahan_comp"), lr=group["lr"], beta1=group["beta1"],
                beta2=group["beta2"], beta3=group["beta3"], eps=group["eps"], weight_decay=group["weight_decay"],
                step=step, decouple_lr=group["decouple_lr"], max_lr=group["max_lr"], kahan_sum=group["kahan_sum"],
-               foreach=False, triton=group["triton"], gradient_release=gradient_release,
+               foreach=False, triton=True, gradient_release=gradient_release,
                optimizer_accumulation=accumulate, _groups=self._hip_groups)

@@ -64,50 +64,61 @@ def _beta_hat(beta: float, t: int) -> float:
     return (bt - beta) / (bt - 1)
 
 
+def step_scalars(name: str, h: dict, t: int | None, kahan_sum: bool, accumulate: bool):
+    """The scalar arguments of one step, in the order the C entry points take them after
+    ``dtype``: formed from the raw hyper-parameters ``h`` the way the reference's functional
+    forms do (optimi/adam.py:260-273, lion.py:226-235, stableadamw.py:326-332, adan.py:289-309).
+    ``t`` is the already advanced step count (None for Lion)."""
+    lr, wd = h["lr"], h.get("weight_decay", 0.0)
+    flags = (KAHAN if kahan_sum else 0) | (0 if accumulate else UPDATE)
+    ratio = lr / h["max_lr"] if h.get("decouple_lr") else lr  # lr, or lr/max_lr when fully decoupled
+    if name in ("adam", "adamw"):
+        b1, b2 = h.get("betas", (0.9, 0.99))
+        b1h, b2h = _beta_hat(b1, t), _beta_hat(b2, t)
+        decoupled = name == "adamw" or h.get("decouple_wd", False) or h.get("decouple_lr", False)
+        w = 1 - ratio * wd if (wd != 0 and decoupled) else wd
+        return (lr, 1 - b1h, b2h, 1 - b2h, w, h["eps"], flags | (DECOUPLE_WD if decoupled else 0))
+    if name == "lion":
+        b1, b2 = h.get("betas", (0.9, 0.99))
+        w = 1 - ratio * wd if wd != 0 else 0.0
+        return (lr, 1 - b1, 1 - b2, w, flags)
+    if name == "stableadamw":
+        b1, b2 = h.get("betas", (0.9, 0.99))
+        b1h, b2h = _beta_hat(b1, t), _beta_hat(b2, t)
+        dl = bool(h.get("decouple_lr"))
+        return (lr, 1 - b1h, b2h, 1 - b2h, wd, h["eps"], h["max_lr"] if dl else 0.0, flags | (DECOUPLE_LR if dl else 0))
+    if name == "adan":
+        b1, b2, b3 = h.get("betas", (0.98, 0.92, 0.99))
+        b1h, b2h, b3h = _beta_hat(b1, t), _beta_hat(b2, t), _beta_hat(b3, t)
+        w = 1 + ratio * wd if wd != 0 else 0.0  # the class path is always Adan-style (adan.py:181-203)
+        return (lr, 1 - b1h, b2, 1 - b2h, b3h, 1 - b3h, h["eps"], w, flags)
+    raise ValueError(name)
+
+
+# state buffers each C entry point takes between ``grad`` and ``kahan_comp``
+STATE_ORDER = {
+    "adam": ("exp_avg", "exp_avg_sq"),
+    "adamw": ("exp_avg", "exp_avg_sq"),
+    "lion": ("exp_avg",),
+    "stableadamw": ("exp_avg", "exp_avg_sq"),
+    "adan": ("exp_avg", "exp_avg_diff", "exp_avg_sq", "prev_grad"),
+}
+
+
 class ScalarRun(ForLoopRun):
     """Same state handling as ``ForLoopRun``; the arithmetic is the C emulator's."""
 
     def _call(self, idxs, grads, step, accumulate):
         L = lib()
-        h = self.hyper
-        lr, wd = h["lr"], h.get("weight_decay", 0.0)
-        flags = (KAHAN if self.kahan_sum else 0) | (0 if accumulate else UPDATE)
+        t = None
         if self.name != "lion":
             step.add_(1)
             t = int(step.item())
-        ratio = lr / h["max_lr"] if h.get("decouple_lr") else lr  # lr, or lr/max_lr when fully decoupled
+        scalars = step_scalars(self.name, self.hyper, t, self.kahan_sum, accumulate)
+        fn = {"adam": L.optimi_ref_adam, "adamw": L.optimi_ref_adam, "lion": L.optimi_ref_lion,
+              "stableadamw": L.optimi_ref_stableadamw, "adan": L.optimi_ref_adan}[self.name]
         for i, g in zip(idxs, grads):
             st = self._ensure_state(i, g)
             p = self.params[i]
-            n, dt = p.numel(), _dt(p)
-            if self.name in ("adam", "adamw"):
-                b1, b2 = h.get("betas", (0.9, 0.99))
-                b1h, b2h = _beta_hat(b1, t), _beta_hat(b2, t)
-                decoupled = self.name == "adamw" or h.get("decouple_wd", False) or h.get("decouple_lr", False)
-                w = wd
-                if wd != 0 and decoupled:  # adam.py:269-273
-                    w = 1 - ratio * wd
-                L.optimi_ref_adam(_ptr(p), _ptr(g), _ptr(st["exp_avg"]), _ptr(st["exp_avg_sq"]), _ptr(st["kahan_comp"]),
-                                  n, dt, lr, 1 - b1h, b2h, 1 - b2h, w, h["eps"],
-                                  flags | (DECOUPLE_WD if decoupled else 0))
-            elif self.name == "lion":
-                b1, b2 = h.get("betas", (0.9, 0.99))
-                w = 1 - ratio * wd if wd != 0 else 0.0  # lion.py:226-231
-                L.optimi_ref_lion(_ptr(p), _ptr(g), _ptr(st["exp_avg"]), _ptr(st["kahan_comp"]), n, dt, lr, 1 - b1,
-                                  1 - b2, w, flags)
-            elif self.name == "stableadamw":
-                b1, b2 = h.get("betas", (0.9, 0.99))
-                b1h, b2h = _beta_hat(b1, t), _beta_hat(b2, t)
-                dl = bool(h.get("decouple_lr"))
-                L.optimi_ref_stableadamw(_ptr(p), _ptr(g), _ptr(st["exp_avg"]), _ptr(st["exp_avg_sq"]),
-                                         _ptr(st["kahan_comp"]), n, dt, lr, 1 - b1h, b2h, 1 - b2h, wd, h["eps"],
-                                         h["max_lr"] if dl else 0.0, flags | (DECOUPLE_LR if dl else 0))
-            elif self.name == "adan":
-                b1, b2, b3 = h.get("betas", (0.98, 0.92, 0.99))
-                b1h, b2h, b3h = _beta_hat(b1, t), _beta_hat(b2, t), _beta_hat(b3, t)
-                w = 1 + ratio * wd if wd != 0 else 0.0  # adan.py:300-309; the class path is always Adan-style
-                L.optimi_ref_adan(_ptr(p), _ptr(g), _ptr(st["exp_avg"]), _ptr(st["exp_avg_diff"]),
-                                  _ptr(st["exp_avg_sq"]), _ptr(st["prev_grad"]), _ptr(st["kahan_comp"]), n, dt, lr,
-                                  1 - b1h, b2, 1 - b2h, b3h, 1 - b3h, h["eps"], w, flags)
-            else:
-                raise ValueError(self.name)
+            bufs = [_ptr(st[k]) for k in STATE_ORDER[self.name]]
+            fn(_ptr(p), _ptr(g), *bufs, _ptr(st["kahan_comp"]), p.numel(), _dt(p), *scalars)

@@ -1,0 +1,61 @@
+"""Drives the HIP library through its C ABI with the ``step`` / ``step_param`` interface of
+``oracle.forloop.ForLoopRun``, so the same replay code feeds the oracle and the kernels.
+
+torch only provides device memory and the stream here: every launch goes through
+``optimi_amd.cabi`` (ctypes on ``liboptimi_hip.so``).  Step scalars come from
+``oracle.scalar.step_scalars`` – the prologue the golden fixtures pin.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from optimi_amd import cabi
+from oracle.forloop import ForLoopRun
+from oracle.scalar import STATE_ORDER, step_scalars
+
+DT = {torch.float32: cabi.F32, torch.bfloat16: cabi.BF16}
+
+
+def _addr(t):
+    return None if t is None else t.data_ptr()
+
+
+class HipRun(ForLoopRun):
+    """``multi=True``: whole-list entry points (one launch); False: per-tensor entry points."""
+
+    def __init__(self, name, params, *, multi=True, **kw):
+        super().__init__(name, params, **kw)
+        self.multi = multi
+        self.group = cabi.Group()
+        self.entry = "adam" if name == "adamw" else name
+
+    def _stream(self):
+        return torch.cuda.current_stream().cuda_stream
+
+    def _call(self, idxs, grads, step, accumulate):
+        L = cabi.lib()
+        t = None
+        if self.name != "lion":
+            step.add_(1)
+            t = int(step.item())
+        scalars = step_scalars(self.name, self.hyper, t, self.kahan_sum, accumulate)
+        sts = [self._ensure_state(i, g) for i, g in zip(idxs, grads)]
+        ps = [self.params[i] for i in idxs]
+        if not ps:
+            return
+        dt = DT[ps[0].dtype]
+        if self.multi and not self.gradient_release:
+            cols = [cabi.ptr_array(_addr(p) for p in ps), cabi.ptr_array(_addr(g) for g in grads)]
+            cols += [cabi.ptr_array(_addr(s[k]) for s in sts) for k in STATE_ORDER[self.name]]
+            cols.append(cabi.ptr_array(_addr(s["kahan_comp"]) for s in sts))
+            fn = getattr(L, f"optimi_hip_{self.entry}_multi")
+            rc = fn(self.group.handle, len(ps), *cols, cabi.i64_array(p.numel() for p in ps), dt, *scalars, self._stream())
+            cabi.check(rc, fn.__name__)
+        else:
+            fn = getattr(L, f"optimi_hip_{self.entry}_single")
+            lead = (self.group.handle,) if self.entry == "stableadamw" else ()
+            for p, g, s in zip(ps, grads, sts):
+                bufs = [_addr(s[k]) for k in STATE_ORDER[self.name]]
+                rc = fn(*lead, _addr(p), _addr(g), *bufs, _addr(s["kahan_comp"]), p.numel(), dt, *scalars, self._stream())
+                cabi.check(rc, fn.__name__)

@@ -1,0 +1,60 @@
+"""The C-ABI library loads without a GPU and exports every function include/optimi_hip.h
+declares.  No compute entry point is called here."""
+
+import ctypes
+import os
+import re
+
+from optimi_amd import cabi
+
+HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "optimi_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(optimi_hip_\w+)\s*\(", text)))
+
+
+def test_header_and_prototypes_agree():
+    assert declared_functions() == sorted(cabi.PROTOTYPES)
+
+
+def test_every_declared_symbol_is_exported():
+    L = cabi.lib()
+    for name in declared_functions():
+        assert getattr(L, name) is not None, name
+
+
+def test_error_strings_and_constants():
+    L = cabi.lib()
+    assert L.optimi_hip_version() >= 1000
+    assert L.optimi_hip_error_string(0) == b"success"
+    for code in range(-7, 0):
+        msg = L.optimi_hip_error_string(code)
+        assert msg.startswith(b"optimi_hip:"), (code, msg)
+    assert L.optimi_hip_chunk_elems(cabi.BF16) == 8192
+    assert L.optimi_hip_chunk_elems(cabi.F32) == 4096
+    assert L.optimi_hip_chunk_elems(7) < 0
+    # the flag values the Python side uses are the header's
+    text = open(HEADER).read()
+    for name, val in (("KAHAN", cabi.KAHAN), ("UPDATE", cabi.UPDATE), ("DECOUPLE_WD", cabi.DECOUPLE_WD),
+                      ("ADAM_WD", cabi.ADAM_WD), ("DECOUPLE_LR", cabi.DECOUPLE_LR)):
+        assert re.search(rf"OPTIMI_{name}\s*=\s*{val}\b", text), name
+
+
+def test_null_group_is_rejected_before_any_device_work():
+    L = cabi.lib()
+    assert L.optimi_hip_group_create(None) == -1
+    assert L.optimi_hip_group_destroy(None) == 0
+    nothing = (ctypes.c_void_p * 1)()
+    sizes = (ctypes.c_int64 * 1)(0)
+    rc = L.optimi_hip_adam_multi(None, 0, nothing, nothing, nothing, nothing, nothing, sizes, cabi.F32,
+                                 1e-3, 0.1, 0.9, 0.1, 0.0, 1e-6, cabi.UPDATE, None)
+    assert rc == -1
+    # argument checks of the per-tensor entry points run before any launch
+    assert L.optimi_hip_adam_single(None, None, None, None, None, -1, cabi.F32, 1e-3, 0.1, 0.9, 0.1, 0.0, 1e-6, 2, None) == -2
+    assert L.optimi_hip_adam_single(None, None, None, None, None, 8, 9, 1e-3, 0.1, 0.9, 0.1, 0.0, 1e-6, 2, None) == -3
+    assert L.optimi_hip_adam_single(None, None, None, None, None, 8, cabi.F32, 1e-3, 0.1, 0.9, 0.1, 0.0, 1e-6, 2, None) == -1
+    assert L.optimi_hip_adam_single(None, None, None, None, None, 0, cabi.F32, 1e-3, 0.1, 0.9, 0.1, 0.0, 1e-6, 2, None) == 0
+    assert L.optimi_hip_copy_probe(None, None, 16, None) == -1

@@ -1,0 +1,56 @@
+"""HIP kernels against the golden vectors the reference wrote (tests/golden/*.npz).
+
+Each fixture is replayed twice through the C ABI – once with the whole-list entry points,
+once with the per-tensor entry points – and every snapshot (params and all states after
+steps 1, 3 and the last) is compared with what the reference's for-loop path produced.
+
+Bar: bf16 tensors bit-exact, except StableAdamW, whose per-tensor mean is summed in a
+different order than torch's (<= 1 bf16 ulp there; the Kahan buffer is judged in units of
+the parameter's ulp).  fp32 tensors: |a-b| <= 1e-6 * max(|a|, |b|, floor); torch's CPU sqrt
+is only faithfully rounded, so fp32 cannot be bit-exact.  The floor covers elements that
+cancel towards zero: 1e-3 for parameters (one step moves a parameter by about lr = 1e-3, so
+its rounding error is judged against that distance, i.e. |a-b| <= 1e-9 near zero) and 1e-12
+for the moment states.
+"""
+
+import functools
+
+import pytest
+import torch
+
+import golden_util as G
+
+pytestmark = pytest.mark.gpu
+
+FP32_REL = 1e-6
+FP32_FLOOR_PARAM = 1e-3
+FP32_FLOOR_STATE = 1e-12
+
+
+def compare_snapshot(name, key, got, want, param_want=None):
+    if want.dtype == torch.bfloat16:
+        ulp = G.bf16_ulp_diff(got, want)
+        if "stableadamw" not in name:
+            assert int(ulp.max()) == 0, f"{name} {key}: {int((ulp > 0).sum())} of {ulp.numel()} differ, max {int(ulp.max())} ulp"
+        elif ".kahan_comp." in key:
+            err = (got.float() - want.float()).abs() / G.bf16_ulp_of(param_want)
+            assert float(err.max()) <= 1.0, f"{name} {key}: Kahan buffer off by {float(err.max())} param ulps"
+        else:
+            assert int(ulp.max()) <= 1, f"{name} {key}: max {int(ulp.max())} ulp"
+    else:
+        rel = G.fp32_rel_err(got, want, FP32_FLOOR_PARAM if ".param." in key else FP32_FLOOR_STATE)
+        assert float(rel.max()) <= FP32_REL, f"{name} {key}: rel err {float(rel.max())}"
+
+
+@pytest.mark.parametrize("multi", [True, False], ids=["multi", "single"])
+@pytest.mark.parametrize("name", G.case_names())
+def test_fixture(name, multi, hip_device):
+    from hip_engine import HipRun
+
+    fx = G.load(name)
+    out = G.replay(name, fx, functools.partial(HipRun, multi=multi), device=hip_device)
+    wanted = [k for k in fx if k.startswith("out.")]
+    assert sorted(out) == sorted(wanted)
+    for key in wanted:
+        step, _, idx = key.split(".")[1], key.split(".")[2], key.split(".")[3]
+        compare_snapshot(name, key, out[key], fx[key], fx.get(f"out.{step}.param.{idx}"))
