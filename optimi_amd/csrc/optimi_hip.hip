@@ -1,11 +1,14 @@
 // Fused optimizer-step kernels for MI355X (gfx950) and the C ABI around them.
 //
 // Every kernel here is a bandwidth-bound stream over a handful of equally sized arrays
-// (param, grad, moments, Kahan buffer).  One workgroup of 256 lanes covers one chunk of
-// 16 KiB per array: each lane issues kUnroll 16-byte loads per array before the first
-// use, does the arithmetic in fp32 registers, and writes 16-byte stores back in place.
-// A whole parameter list runs as ONE launch: a chunk map (chunk -> tensor) and a tensor
-// table (pointers, size, first chunk) tell each workgroup where it works.
+// (param, grad, moments, Kahan buffer).  Tensors are cut into chunks of 16 KiB per array;
+// kSub workgroups of kThreads lanes share a chunk, each lane issuing kUnroll 16-byte loads
+// per array before the first use, doing the arithmetic in fp32 registers and writing
+// 16-byte stores back in place.  A whole parameter list runs as ONE launch: a chunk map
+// (chunk -> tensor) and a tensor table (pointers, size, first chunk) tell each workgroup
+// where it works.  How many workgroups a CU holds at once is throttled with a dummy
+// dynamic-LDS request (see throttle_lds): with up to thirteen concurrent streams HBM runs
+// best when only a few tens of KiB per CU are in flight.
 //
 // Arithmetic contract.  Results follow optimi's PyTorch for-loop path
 // (optimi/adam.py:354-396, lion.py:301-338, stableadamw.py:421-472, adan.py:405-469),
@@ -23,14 +26,26 @@
 #include <cstdlib>
 #include <cstring>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 #include "optimi_hip.h"
 
 namespace {
 
-constexpr int kThreads = 256;   // lanes per workgroup (4 wavefronts of 64)
-constexpr int kUnroll = 4;      // 16-byte vectors per lane per array
+#ifndef OPTIMI_THREADS
+#define OPTIMI_THREADS 64
+#endif
+#ifndef OPTIMI_UNROLL
+#define OPTIMI_UNROLL 1
+#endif
+constexpr int kThreads = OPTIMI_THREADS;  // lanes per workgroup
+constexpr int kUnroll = OPTIMI_UNROLL;    // 16-byte vectors per lane per array
+constexpr int kChunkBytes = 16384;        // bytes per array per chunk: the granule of the chunk map
+constexpr int kSub = kChunkBytes / (kThreads * kUnroll * 16);  // workgroups per chunk
+static_assert(kSub >= 1 && kSub * kThreads * kUnroll * 16 == kChunkBytes, "workgroup tile must divide the chunk");
+static_assert(kThreads % 64 == 0 && kThreads <= 1024, "whole wavefronts");
+constexpr int kReduceThreads = 256;       // lanes of the per-tensor finalize workgroup
 constexpr int kMaxArrays = 7;   // Adan: p g m diff sq prev kahan
 constexpr int kAbiVersion = 1000;
 
@@ -38,57 +53,70 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
+// Pointers come out of the tensor table as plain addresses; telling the compiler they are
+// global memory gets global_load/global_store instead of flat accesses.
+#define OPTIMI_GLOBAL __attribute__((address_space(1)))
+__device__ __forceinline__ u32x4 load16(const void* base, int64_t byte_off) {
+  return __builtin_nontemporal_load((const OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
+}
+__device__ __forceinline__ void store16(void* base, int64_t byte_off, u32x4 v) {
+  __builtin_nontemporal_store(v, (OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
+}
+
+// Element math runs on pairs of neighbouring elements (f32x2): one v_cvt_pk_bf16_f32 then
+// rounds two values.  With packed fp32 ops disabled the pair arithmetic is two scalar ops.
+__device__ __forceinline__ f32x2 splat(float x) { return f32x2{x, x}; }
+__device__ __forceinline__ f32x2 fma2(f32x2 a, f32x2 b, f32x2 c) { return f32x2{fmaf(a.x, b.x, c.x), fmaf(a.y, b.y, c.y)}; }
+#ifdef OPTIMI_PROBE_FAST  // measurement only: how much the exact sqrt/divide sequences cost
+__device__ __forceinline__ f32x2 sqrt2(f32x2 a) { return f32x2{__builtin_amdgcn_sqrtf(a.x), __builtin_amdgcn_sqrtf(a.y)}; }
+__device__ __forceinline__ f32x2 div2(f32x2 a, f32x2 b) { return f32x2{a.x * __builtin_amdgcn_rcpf(b.x), a.y * __builtin_amdgcn_rcpf(b.y)}; }
+#else
+__device__ __forceinline__ f32x2 sqrt2(f32x2 a) { return f32x2{sqrtf(a.x), sqrtf(a.y)}; }
+__device__ __forceinline__ f32x2 div2(f32x2 a, f32x2 b) { return f32x2{a.x / b.x, a.y / b.y}; }
+#endif
+
 // ------------------------------------------------------------------------------------
 // dtype policies
 // ------------------------------------------------------------------------------------
 struct F32 {
-  static constexpr int kVec = 4;  // elements per 16-byte vector
+  static constexpr int kVec = 4;    // elements per 16-byte vector
+  static constexpr int kPairs = 2;  // element pairs per vector
   static constexpr int kElemBytes = 4;
-  static constexpr int kDtype = OPTIMI_F32;
-  static constexpr bool kLowPrecision = false;
-  __device__ static __forceinline__ float R(float x) { return x; }
-  __device__ static __forceinline__ void unpack(const u32x4& r, float* f) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(r[i]);
+  __device__ static __forceinline__ f32x2 R2(f32x2 x) { return x; }
+  __device__ static __forceinline__ void unpack(const u32x4& r, f32x2* f) {
+    f[0] = f32x2{__uint_as_float(r[0]), __uint_as_float(r[1])};
+    f[1] = f32x2{__uint_as_float(r[2]), __uint_as_float(r[3])};
   }
-  __device__ static __forceinline__ u32x4 pack(const float* f) {
-    u32x4 r;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) r[i] = __float_as_uint(f[i]);
-    return r;
+  __device__ static __forceinline__ u32x4 pack(const f32x2* f) {
+    return u32x4{__float_as_uint(f[0].x), __float_as_uint(f[0].y), __float_as_uint(f[1].x), __float_as_uint(f[1].y)};
   }
-  __device__ static __forceinline__ float load1(const void* p, int64_t i) { return ((const float*)p)[i]; }
-  __device__ static __forceinline__ void store1(void* p, int64_t i, float x) { ((float*)p)[i] = x; }
+  __device__ static __forceinline__ float load1(const void* p, int64_t i) { return ((const OPTIMI_GLOBAL float*)(uintptr_t)p)[i]; }
+  __device__ static __forceinline__ void store1(void* p, int64_t i, float x) { ((OPTIMI_GLOBAL float*)(uintptr_t)p)[i] = x; }
 };
 
 struct BF16 {
   static constexpr int kVec = 8;
+  static constexpr int kPairs = 4;
   static constexpr int kElemBytes = 2;
-  static constexpr int kDtype = OPTIMI_BF16;
-  static constexpr bool kLowPrecision = true;
-  // round-to-nearest-even to bf16, returned widened (v_cvt_pk_bf16_f32 + shift on gfx950)
-  __device__ static __forceinline__ float R(float x) { return (float)(__bf16)x; }
-  __device__ static __forceinline__ void unpack(const u32x4& r, float* f) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      f[2 * i] = __uint_as_float(r[i] << 16);
-      f[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
-    }
+  __device__ static __forceinline__ f32x2 widen(uint32_t two) {  // two packed bf16 -> two floats
+    return f32x2{__uint_as_float(two << 16), __uint_as_float(two & 0xffff0000u)};
   }
-  __device__ static __forceinline__ u32x4 pack(const float* f) {  // f[] hold exact bf16 values
-    u32x4 r;
+  __device__ static __forceinline__ uint32_t narrow(f32x2 x) {  // round-to-nearest-even, v_cvt_pk_bf16_f32
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+  }
+  __device__ static __forceinline__ f32x2 R2(f32x2 x) { return widen(narrow(x)); }
+  __device__ static __forceinline__ void unpack(const u32x4& r, f32x2* f) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      f32x2 v = {f[2 * i], f[2 * i + 1]};
-      r[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-    }
-    return r;
+    for (int i = 0; i < 4; ++i) f[i] = widen(r[i]);
+  }
+  __device__ static __forceinline__ u32x4 pack(const f32x2* f) {  // f[] hold exact bf16 values
+    return u32x4{narrow(f[0]), narrow(f[1]), narrow(f[2]), narrow(f[3])};
   }
   __device__ static __forceinline__ float load1(const void* p, int64_t i) {
-    return __uint_as_float((uint32_t)((const uint16_t*)p)[i] << 16);
+    return __uint_as_float((uint32_t)((const OPTIMI_GLOBAL uint16_t*)(uintptr_t)p)[i] << 16);
   }
   __device__ static __forceinline__ void store1(void* p, int64_t i, float x) {
-    ((uint16_t*)p)[i] = (uint16_t)(__float_as_uint(x) >> 16);
+    ((OPTIMI_GLOBAL uint16_t*)(uintptr_t)p)[i] = (uint16_t)(__float_as_uint(x) >> 16);
   }
 };
 
@@ -115,32 +143,35 @@ struct Lerp {
   float coef;
   uint32_t small;
 };
-__device__ __forceinline__ float lerp_apply(float start, float end, const Lerp& l) {
-  float d = end - start;
-  return fmaf(l.coef, d, l.small ? start : end);
+__device__ __forceinline__ f32x2 lerp2(f32x2 start, f32x2 end, const Lerp& l) {
+  f32x2 d = end - start;
+  return fma2(splat(l.coef), d, l.small ? start : end);
 }
 
+// param += kahan; kahan += (old param - new param)
 template <class DT>
-__device__ __forceinline__ void kahan_commit(float& p, float& k) {
-  float old = p;
-  p = DT::R(old + k);
-  float err = DT::R(old - p);
-  k = DT::R(k + err);
+__device__ __forceinline__ void kahan_commit(f32x2& p, f32x2& k) {
+  f32x2 old = p;
+  p = DT::R2(old + k);
+  f32x2 err = DT::R2(old - p);
+  k = DT::R2(k + err);
 }
 
 constexpr uint32_t bit(int i) { return 1u << i; }
 
 // ------------------------------------------------------------------------------------
-// element functions.  x[] is indexed by array slot; each Op names its slots.
+// element functions on pairs.  x[] is indexed by array slot; each Op names its slots.
+// KAHAN / UPDATE / WD are compile-time so the inner code is branch-free; UPDATE=false is the
+// accumulate-only step, which touches neither the parameter nor the Kahan buffer.
 // ------------------------------------------------------------------------------------
 struct AdamScalars {
   Lerp l1;
   float wd, wd_alpha, b2h, b2c, eps_d, neg_lr;
-  uint32_t wd_mode;  // 0 none, 1 decoupled (p *= wd), 2 L2 (g += wd_alpha * p)
 };
 
 // slots: 0 param, 1 grad, 2 exp_avg, 3 exp_avg_sq, 4 kahan_comp     optimi/adam.py:354-396
-template <class DT_, bool KAHAN, bool UPDATE>
+// WD: 0 none, 1 decoupled (p *= wd), 2 L2 (g += wd_alpha * p)
+template <class DT_, bool KAHAN, bool UPDATE, int WD>
 struct AdamOp {
   using DT = DT_;
   using Scalars = AdamScalars;
@@ -149,27 +180,25 @@ struct AdamOp {
   static constexpr uint32_t kStore = UPDATE ? (bit(0) | bit(2) | bit(3) | (KAHAN ? bit(4) : 0)) : (bit(2) | bit(3));
   static constexpr bool kReduce = false;
   __device__ static __forceinline__ void prepare(Scalars&, int) {}
-  __device__ static __forceinline__ void elem(float* x, const Scalars& s, float&) {
-    float p = x[0], g = x[1], m = x[2], v = x[3];
-    if (UPDATE) {
-      if (s.wd_mode == 1) p = DT::R(p * s.wd);
-      else if (s.wd_mode == 2) g = DT::R(fmaf(p, s.wd_alpha, g));
-    }
-    m = DT::R(lerp_apply(m, g, s.l1));
-    v = DT::R(v * s.b2h);
-    v = DT::R(fmaf(s.b2c * g, g, v));
+  __device__ static __forceinline__ void elem(f32x2* x, const Scalars& s, f32x2&) {
+    f32x2 p = x[0], g = x[1], m = x[2], v = x[3];
+    if (UPDATE && WD == 1) p = DT::R2(p * s.wd);
+    if (UPDATE && WD == 2) g = DT::R2(fma2(p, splat(s.wd_alpha), g));
+    m = DT::R2(lerp2(m, g, s.l1));
+    v = DT::R2(v * s.b2h);
+    v = DT::R2(fma2(g * s.b2c, g, v));
     x[2] = m;
     x[3] = v;
     if (UPDATE) {
-      float d = DT::R(sqrtf(v));
-      d = DT::R(d + s.eps_d);
+      f32x2 d = DT::R2(sqrt2(v));
+      d = DT::R2(d + s.eps_d);
       if (KAHAN) {
-        float k = x[4];
-        k = DT::R(k + (s.neg_lr * m) / d);
+        f32x2 k = x[4];
+        k = DT::R2(k + div2(m * s.neg_lr, d));
         kahan_commit<DT>(p, k);
         x[4] = k;
       } else {
-        p = DT::R(p + (s.neg_lr * m) / d);
+        p = DT::R2(p + div2(m * s.neg_lr, d));
       }
       x[0] = p;
     }
@@ -179,11 +208,11 @@ struct AdamOp {
 struct LionScalars {
   Lerp l1, l2;
   float wd, neg_lr_d;
-  uint32_t do_wd;
 };
 
 // slots: 0 param, 1 grad, 2 exp_avg, 3 kahan_comp                  optimi/lion.py:301-338
-template <class DT_, bool KAHAN, bool UPDATE>
+// WD: 0 none, 1 decoupled
+template <class DT_, bool KAHAN, bool UPDATE, int WD>
 struct LionOp {
   using DT = DT_;
   using Scalars = LionScalars;
@@ -192,24 +221,25 @@ struct LionOp {
   static constexpr uint32_t kStore = UPDATE ? (bit(0) | bit(2) | (KAHAN ? bit(3) : 0)) : bit(2);
   static constexpr bool kReduce = false;
   __device__ static __forceinline__ void prepare(Scalars&, int) {}
-  __device__ static __forceinline__ void elem(float* x, const Scalars& s, float&) {
-    float p = x[0], g = x[1], m = x[2];
-    float u = 0.0f;
+  __device__ static __forceinline__ float sign1(float c) { return (float)((c > 0.0f) - (c < 0.0f)); }
+  __device__ static __forceinline__ void elem(f32x2* x, const Scalars& s, f32x2&) {
+    f32x2 p = x[0], g = x[1], m = x[2];
+    f32x2 u = splat(0.0f);
     if (UPDATE) {
-      if (s.do_wd) p = DT::R(p * s.wd);
-      float c = DT::R(lerp_apply(m, g, s.l1));
-      u = (float)((c > 0.0f) - (c < 0.0f));
+      if (WD == 1) p = DT::R2(p * s.wd);
+      f32x2 c = DT::R2(lerp2(m, g, s.l1));
+      u = f32x2{sign1(c.x), sign1(c.y)};
     }
-    m = DT::R(lerp_apply(m, g, s.l2));
+    m = DT::R2(lerp2(m, g, s.l2));
     x[2] = m;
     if (UPDATE) {
       if (KAHAN) {
-        float k = x[3];
-        k = DT::R(fmaf(u, s.neg_lr_d, k));
+        f32x2 k = x[3];
+        k = DT::R2(fma2(u, splat(s.neg_lr_d), k));
         kahan_commit<DT>(p, k);
         x[3] = k;
       } else {
-        p = DT::R(fmaf(u, s.neg_lr_d, p));
+        p = DT::R2(fma2(u, splat(s.neg_lr_d), p));
       }
       x[0] = p;
     }
@@ -221,7 +251,8 @@ struct StableP1Scalars {
   float b2h, b2c, eps_sq_d;
 };
 
-// StableAdamW pass 1: moments and sum of g^2/max(v, eps^2).  Slots as Adam.   stableadamw.py:442-447
+// StableAdamW pass 1: moments and g^2/max(v, eps^2) per element (summed by the kernel).
+// Slots as Adam.                                                optimi/stableadamw.py:442-447
 template <class DT_, bool UPDATE>
 struct StablePass1Op {
   using DT = DT_;
@@ -231,18 +262,17 @@ struct StablePass1Op {
   static constexpr uint32_t kStore = bit(2) | bit(3);
   static constexpr bool kReduce = UPDATE;
   __device__ static __forceinline__ void prepare(Scalars&, int) {}
-  __device__ static __forceinline__ void elem(float* x, const Scalars& s, float& acc) {
-    float g = x[1], m = x[2], v = x[3];
-    m = DT::R(lerp_apply(m, g, s.l1));
-    v = DT::R(v * s.b2h);
-    v = DT::R(fmaf(s.b2c * g, g, v));
+  __device__ static __forceinline__ void elem(f32x2* x, const Scalars& s, f32x2& q) {
+    f32x2 g = x[1], m = x[2], v = x[3];
+    m = DT::R2(lerp2(m, g, s.l1));
+    v = DT::R2(v * s.b2h);
+    v = DT::R2(fma2(g * s.b2c, g, v));
     x[2] = m;
     x[3] = v;
     if (UPDATE) {
-      float q = DT::R(g * g);
-      float mx = v > s.eps_sq_d ? v : s.eps_sq_d;
-      q = DT::R(q / mx);
-      acc += q;
+      q = DT::R2(g * g);
+      f32x2 mx = f32x2{v.x > s.eps_sq_d ? v.x : s.eps_sq_d, v.y > s.eps_sq_d ? v.y : s.eps_sq_d};
+      q = DT::R2(div2(q, mx));
     }
   }
 };
@@ -250,11 +280,11 @@ struct StablePass1Op {
 struct StableP2Scalars {
   const TensorScalars* per_tensor;
   float eps_d, neg_lr, wd;  // neg_lr, wd are filled per tensor by prepare()
-  uint32_t do_wd;
 };
 
-// StableAdamW pass 2: decay with the clipped lr, then the Adam tail.          stableadamw.py:453-472
-template <class DT_, bool KAHAN>
+// StableAdamW pass 2: decay with the clipped lr, then the Adam tail.   stableadamw.py:453-472
+// WD: 0 none, 1 decoupled with the per-tensor factor
+template <class DT_, bool KAHAN, int WD>
 struct StablePass2Op {
   using DT = DT_;
   using Scalars = StableP2Scalars;
@@ -267,18 +297,18 @@ struct StablePass2Op {
     s.neg_lr = t.neg_lr;
     s.wd = t.wd_factor;
   }
-  __device__ static __forceinline__ void elem(float* x, const Scalars& s, float&) {
-    float p = x[0], m = x[2], v = x[3];
-    if (s.do_wd) p = DT::R(p * s.wd);
-    float d = DT::R(sqrtf(v));
-    d = DT::R(d + s.eps_d);
+  __device__ static __forceinline__ void elem(f32x2* x, const Scalars& s, f32x2&) {
+    f32x2 p = x[0], m = x[2], v = x[3];
+    if (WD == 1) p = DT::R2(p * s.wd);
+    f32x2 d = DT::R2(sqrt2(v));
+    d = DT::R2(d + s.eps_d);
     if (KAHAN) {
-      float k = x[4];
-      k = DT::R(k + (s.neg_lr * m) / d);
+      f32x2 k = x[4];
+      k = DT::R2(k + div2(m * s.neg_lr, d));
       kahan_commit<DT>(p, k);
       x[4] = k;
     } else {
-      p = DT::R(p + (s.neg_lr * m) / d);
+      p = DT::R2(p + div2(m * s.neg_lr, d));
     }
     x[0] = p;
   }
@@ -287,11 +317,11 @@ struct StablePass2Op {
 struct AdanScalars {
   Lerp l1, l2;
   float b2, b3h, b3c, eps_d, neg_lr, neg_lr_b2, wd;
-  uint32_t wd_mode;  // 0 none, 1 Adam style (p *= wd before), 2 Adan style (p /= wd after)
 };
 
 // slots: 0 param, 1 grad, 2 exp_avg, 3 exp_avg_diff, 4 exp_avg_sq, 5 prev_grad, 6 kahan   adan.py:405-469
-template <class DT_, bool KAHAN, bool UPDATE>
+// WD: 0 none, 1 Adam style (p *= wd before the step), 2 Adan style (p /= wd after it)
+template <class DT_, bool KAHAN, bool UPDATE, int WD>
 struct AdanOp {
   using DT = DT_;
   using Scalars = AdanScalars;
@@ -301,35 +331,35 @@ struct AdanOp {
   static constexpr uint32_t kStore = kState | (UPDATE ? (bit(0) | (KAHAN ? bit(6) : 0)) : 0);
   static constexpr bool kReduce = false;
   __device__ static __forceinline__ void prepare(Scalars&, int) {}
-  __device__ static __forceinline__ void elem(float* x, const Scalars& s, float&) {
-    float p = x[0], g = x[1], m = x[2], df = x[3], n = x[4], pg = x[5];
-    pg = DT::R(pg + g);
-    m = DT::R(lerp_apply(m, g, s.l1));
-    df = DT::R(lerp_apply(df, pg, s.l2));
-    pg = DT::R(pg * s.b2);
-    pg = DT::R(pg + g);
-    n = DT::R(n * s.b3h);
-    n = DT::R(fmaf(s.b3c * pg, pg, n));
-    pg = DT::R(g * -1.0f);
+  __device__ static __forceinline__ void elem(f32x2* x, const Scalars& s, f32x2&) {
+    f32x2 p = x[0], g = x[1], m = x[2], df = x[3], n = x[4], pg = x[5];
+    pg = DT::R2(pg + g);
+    m = DT::R2(lerp2(m, g, s.l1));
+    df = DT::R2(lerp2(df, pg, s.l2));
+    pg = DT::R2(pg * s.b2);
+    pg = DT::R2(pg + g);
+    n = DT::R2(n * s.b3h);
+    n = DT::R2(fma2(pg * s.b3c, pg, n));
+    pg = DT::R2(g * -1.0f);
     x[2] = m;
     x[3] = df;
     x[4] = n;
     x[5] = pg;
     if (UPDATE) {
-      float d = DT::R(sqrtf(n));
-      d = DT::R(d + s.eps_d);
-      if (s.wd_mode == 1) p = DT::R(p * s.wd);
+      f32x2 d = DT::R2(sqrt2(n));
+      d = DT::R2(d + s.eps_d);
+      if (WD == 1) p = DT::R2(p * s.wd);
       if (KAHAN) {
-        float k = x[6];
-        k = DT::R(k + (s.neg_lr * m) / d);
-        k = DT::R(k + (s.neg_lr_b2 * df) / d);
+        f32x2 k = x[6];
+        k = DT::R2(k + div2(m * s.neg_lr, d));
+        k = DT::R2(k + div2(df * s.neg_lr_b2, d));
         kahan_commit<DT>(p, k);
         x[6] = k;
       } else {
-        p = DT::R(p + (s.neg_lr * m) / d);
-        p = DT::R(p + (s.neg_lr_b2 * df) / d);
+        p = DT::R2(p + div2(m * s.neg_lr, d));
+        p = DT::R2(p + div2(df * s.neg_lr_b2, d));
       }
-      if (s.wd_mode == 2) p = DT::R(p / s.wd);
+      if (WD == 2) p = DT::R2(div2(p, splat(s.wd)));
       x[0] = p;
     }
   }
@@ -339,49 +369,55 @@ struct AdanOp {
 // the streaming kernel
 // ------------------------------------------------------------------------------------
 template <class DT>
-constexpr int64_t chunk_elems() { return (int64_t)kThreads * DT::kVec * kUnroll; }
+constexpr int64_t chunk_elems() { return kChunkBytes / DT::kElemBytes; }
 
 // Block-wide sum of one double per lane; the result is valid in lane 0 of wave 0.
+template <int THREADS>
 __device__ __forceinline__ double block_sum(double v, double* lds) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  if (THREADS == 64) return v;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (lane == 0) lds[wave] = v;
   __syncthreads();
   if (threadIdx.x == 0) {
     v = lds[0];
 #pragma unroll
-    for (int w = 1; w < kThreads / 64; ++w) v += lds[w];
+    for (int w = 1; w < THREADS / 64; ++w) v += lds[w];
   }
   return v;
 }
 
-// Unpacks one 16-byte vector per loaded array, runs the element function on each lane's
-// elements and writes the stored arrays back to element offset `off` of the tensor.
+// Unpacks one 16-byte vector per loaded array, runs the element function on each pair and
+// writes the stored arrays back to element offset `off` of the tensor.
 template <class Op>
 __device__ __forceinline__ void compute_store(const TensorEntry& e, int64_t off, const u32x4* raw,
                                               const typename Op::Scalars& s, float& acc) {
   using DT = typename Op::DT;
-  constexpr int V = DT::kVec;
+  constexpr int P = DT::kPairs;
   constexpr int A = Op::kArrays;
-  float f[A][V];
+  f32x2 f[A][P];
 #pragma unroll
   for (int a = 0; a < A; ++a)
     if (Op::kLoad & bit(a)) DT::unpack(raw[a], f[a]);
 #pragma unroll
-  for (int i = 0; i < V; ++i) {
-    float x[A];
+  for (int i = 0; i < P; ++i) {
+    f32x2 x[A];
 #pragma unroll
-    for (int a = 0; a < A; ++a) x[a] = (Op::kLoad & bit(a)) ? f[a][i] : 0.0f;
-    Op::elem(x, s, acc);
+    for (int a = 0; a < A; ++a) x[a] = (Op::kLoad & bit(a)) ? f[a][i] : splat(0.0f);
+    f32x2 q = splat(0.0f);
+    Op::elem(x, s, q);
+    if (Op::kReduce) {
+      acc += q.x;
+      acc += q.y;
+    }
 #pragma unroll
     for (int a = 0; a < A; ++a)
       if (Op::kStore & bit(a)) f[a][i] = x[a];
   }
 #pragma unroll
   for (int a = 0; a < A; ++a)
-    if (Op::kStore & bit(a))
-      __builtin_nontemporal_store(DT::pack(f[a]), (u32x4*)((char*)e.ptr[a] + off * DT::kElemBytes));
+    if (Op::kStore & bit(a)) store16(e.ptr[a], off * DT::kElemBytes, DT::pack(f[a]));
 }
 
 template <class Op>
@@ -389,21 +425,22 @@ __device__ __forceinline__ void load_vec(const TensorEntry& e, int64_t off, u32x
   using DT = typename Op::DT;
 #pragma unroll
   for (int a = 0; a < Op::kArrays; ++a)
-    if (Op::kLoad & bit(a))
-      raw[a] = __builtin_nontemporal_load((const u32x4*)((const char*)e.ptr[a] + off * DT::kElemBytes));
+    if (Op::kLoad & bit(a)) raw[a] = load16(e.ptr[a], off * DT::kElemBytes);
 }
 
 template <class Op>
 __device__ __forceinline__ void one_element(const TensorEntry& e, int64_t i, const typename Op::Scalars& s, float& acc) {
   using DT = typename Op::DT;
   constexpr int A = Op::kArrays;
-  float x[A];
+  f32x2 x[A];
 #pragma unroll
-  for (int a = 0; a < A; ++a) x[a] = (Op::kLoad & bit(a)) ? DT::load1(e.ptr[a], i) : 0.0f;
-  Op::elem(x, s, acc);
+  for (int a = 0; a < A; ++a) x[a] = splat((Op::kLoad & bit(a)) ? DT::load1(e.ptr[a], i) : 0.0f);
+  f32x2 q = splat(0.0f);
+  Op::elem(x, s, q);
+  if (Op::kReduce) acc += q.x;
 #pragma unroll
   for (int a = 0; a < A; ++a)
-    if (Op::kStore & bit(a)) DT::store1(e.ptr[a], i, x[a]);
+    if (Op::kStore & bit(a)) DT::store1(e.ptr[a], i, x[a].x);
 }
 
 template <class Op, bool MULTI>
@@ -414,18 +451,21 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
   constexpr int V = DT::kVec;
   constexpr int A = Op::kArrays;
   constexpr int64_t kChunk = chunk_elems<DT>();
+  constexpr int64_t kTile = (int64_t)kThreads * kUnroll * V;  // elements one workgroup covers
 
+  const int64_t chunk_id = blockIdx.x / kSub;
+  const int sub = blockIdx.x % kSub;
   int tensor = 0;
-  if (MULTI) tensor = chunk_map[blockIdx.x];
+  if (MULTI) tensor = chunk_map[chunk_id];
   const TensorEntry& e = MULTI ? table[tensor] : single;
-  const int64_t chunk = (int64_t)blockIdx.x - (MULTI ? e.first_chunk : 0);
-  const int64_t base = chunk * kChunk;
-  const int64_t remain = e.numel - base;
+  const int64_t chunk = chunk_id - (MULTI ? e.first_chunk : 0);
+  const int64_t base = chunk * kChunk + sub * kTile;
+  const int64_t remain = e.numel - base;  // <= 0 for tiles past the end of the tensor's last chunk
   Op::prepare(s, tensor);
 
   float acc = 0.0f;
-  if (e.vec_ok && remain >= kChunk) {
-    // full chunk: every load is issued before the first use
+  if (e.vec_ok && remain >= kTile) {
+    // full tile: every load is issued before the first use
     u32x4 raw[kUnroll][A];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) load_vec<Op>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u]);
@@ -433,7 +473,7 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
     for (int u = 0; u < kUnroll; ++u)
       compute_store<Op>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u], s, acc);
   } else if (e.vec_ok) {
-    // last chunk of a tensor: whole vectors while they fit, then the few leftover elements
+    // end of a tensor: whole vectors while they fit, then the few leftover elements
     const int64_t end = e.numel;
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t off = base + ((int64_t)u * kThreads + threadIdx.x) * V;
@@ -447,13 +487,13 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
     }
   } else {
     // buffers that are not 16-byte aligned: one element at a time
-    const int64_t n = remain < kChunk ? remain : kChunk;
+    const int64_t n = remain < kTile ? remain : kTile;
     for (int64_t i = threadIdx.x; i < n; i += kThreads) one_element<Op>(e, base + i, s, acc);
   }
 
   if (Op::kReduce) {
     __shared__ double lds[kThreads / 64];
-    double total = block_sum((double)acc, lds);
+    double total = block_sum<kThreads>((double)acc, lds);
     if (threadIdx.x == 0) partials[blockIdx.x] = total;
   }
 }
@@ -468,22 +508,22 @@ struct FinalizeArgs {
 };
 
 template <class DT, bool MULTI>
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kReduceThreads)
 stable_finalize_kernel(const TensorEntry* __restrict__ table, const TensorEntry single, const double* __restrict__ partials,
                        TensorScalars* __restrict__ out, FinalizeArgs a) {
   constexpr int64_t kChunk = chunk_elems<DT>();
   const TensorEntry& e = MULTI ? table[blockIdx.x] : single;
-  const int64_t first = MULTI ? e.first_chunk : 0;
-  const int64_t count = (e.numel + kChunk - 1) / kChunk;
+  const int64_t first = (MULTI ? e.first_chunk : 0) * kSub;  // one partial per workgroup of pass 1
+  const int64_t count = (e.numel + kChunk - 1) / kChunk * kSub;
   double v = 0.0;
-  for (int64_t c = threadIdx.x; c < count; c += kThreads) v += partials[first + c];
-  __shared__ double lds[kThreads / 64];
-  double total = block_sum(v, lds);
+  for (int64_t c = threadIdx.x; c < count; c += kReduceThreads) v += partials[first + c];
+  __shared__ double lds[kReduceThreads / 64];
+  double total = block_sum<kReduceThreads>(v, lds);
   if (threadIdx.x == 0) {
     double lr = a.lr;
     if (e.numel > 0) {
-      float ms = DT::R((float)total / (float)e.numel);
-      float rms = DT::R(sqrtf(ms));
+      float ms = DT::R2(splat((float)total / (float)e.numel)).x;
+      float rms = DT::R2(splat(sqrtf(ms))).x;
       double r = (double)rms;
       lr = lr / (r > 1.0 ? r : 1.0);
     }
@@ -495,19 +535,9 @@ stable_finalize_kernel(const TensorEntry* __restrict__ table, const TensorEntry 
   }
 }
 
-__global__ void __launch_bounds__(kThreads) copy_probe_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, int64_t n_vec) {
-  const int64_t base = (int64_t)blockIdx.x * kThreads * kUnroll;
-  u32x4 r[kUnroll];
-#pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    int64_t i = base + (int64_t)u * kThreads + threadIdx.x;
-    if (i < n_vec) r[u] = __builtin_nontemporal_load(src + i);
-  }
-#pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    int64_t i = base + (int64_t)u * kThreads + threadIdx.x;
-    if (i < n_vec) __builtin_nontemporal_store(r[u], dst + i);
-  }
+__global__ void __launch_bounds__(256) copy_probe_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, int64_t n_vec) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n_vec) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 // ------------------------------------------------------------------------------------
@@ -652,7 +682,7 @@ int prepare_tables(optimi_group* g, int n_tensors, const void* const* const* lis
     }
     n_chunks += (numel[t] + chunk - 1) / chunk;
   }
-  if (n_chunks > 0x7fffffff) return OPTIMI_ERR_SIZE;
+  if (n_chunks * kSub > 0x7fffffff) return OPTIMI_ERR_SIZE;
 
   // a group moved to another stream must not overwrite tables a previous launch still reads
   if (g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
@@ -707,41 +737,84 @@ int note_launch(optimi_group* g, hipStream_t stream) {
   return 0;
 }
 
+// Occupancy throttle.  HBM serves this read-modify-write mix best when a CU keeps only about
+// kStreamBudget 16-byte-per-lane vector streams (loads plus stores, counted per wavefront) in
+// flight; more resident wavefronts lower the achieved bandwidth.  The cap is imposed with a
+// dynamic-LDS request that no kernel touches: a CU has 160 KiB of LDS, so asking for L bytes
+// leaves room for floor(160 KiB / L) workgroups.  OPTIMI_HIP_STREAM_BUDGET overrides the budget
+// (0 = no throttle); it is read once.
+constexpr int kStreamBudgetDefault = 86;
+constexpr int kLdsPerCu = 160 * 1024;
+
+int stream_budget() {
+#ifdef OPTIMI_TUNING
+  if (const char* env = std::getenv("OPTIMI_HIP_STREAM_BUDGET")) return (int)std::strtol(env, nullptr, 10);
+#endif
+  static const int value = [] {
+    long v = kStreamBudgetDefault;
+    if (const char* env = std::getenv("OPTIMI_HIP_STREAM_BUDGET")) v = std::strtol(env, nullptr, 10);
+    return (int)(v < 0 ? 0 : v);
+  }();
+  return value;
+}
+
+constexpr int popcount(uint32_t x) { return x ? (int)(x & 1u) + popcount(x >> 1) : 0; }
+
+template <class Op>
+unsigned throttle_lds() {
+  const int budget = stream_budget();
+  if (budget <= 0) return 0;
+  constexpr int streams = (popcount(Op::kLoad) + popcount(Op::kStore)) * kUnroll;
+  int waves = (2 * budget + streams) / (2 * streams);  // round(budget / streams)
+  int wgs = waves / (kThreads / 64);
+  if (wgs < 1) wgs = 1;
+  // midway between "wgs fit" and "wgs + 1 fit", so allocation granularity cannot tip it
+  long lds = (long)(2L * kLdsPerCu / (2 * wgs + 1));
+  if (lds > 65536) lds = 65536;
+  return (unsigned)lds;
+}
+
 template <class Op>
 void launch_multi(optimi_group* g, const typename Op::Scalars& s, hipStream_t stream) {
   TensorEntry none;
   std::memset(&none, 0, sizeof(none));
-  step_kernel<Op, true><<<dim3((unsigned)g->n_chunks), dim3(kThreads), 0, stream>>>(
+  step_kernel<Op, true><<<dim3((unsigned)(g->n_chunks * kSub)), dim3(kThreads), throttle_lds<Op>(), stream>>>(
       (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, none, s, (double*)g->partials.ptr);
 }
 
 template <class Op>
 void launch_single(const TensorEntry& e, const typename Op::Scalars& s, double* partials, hipStream_t stream) {
   const int64_t chunk = chunk_elems<typename Op::DT>();
-  const unsigned blocks = (unsigned)((e.numel + chunk - 1) / chunk);
-  step_kernel<Op, false><<<dim3(blocks), dim3(kThreads), 0, stream>>>(nullptr, nullptr, e, s, partials);
+  const unsigned blocks = (unsigned)((e.numel + chunk - 1) / chunk * kSub);
+  step_kernel<Op, false><<<dim3(blocks), dim3(kThreads), throttle_lds<Op>(), stream>>>(nullptr, nullptr, e, s, partials);
 }
 
-// Runs F<Op>::go() for the Op selected by dtype x kahan x update.
-template <template <class, bool, bool> class OpT, class Fn>
-void dispatch3(int dtype, bool kahan, bool update, Fn&& fn) {
+// Calls fn(Op{}) for the Op selected by dtype x kahan x update x weight-decay mode.  NWD is
+// the number of decay modes the Op family has (modes 0..NWD-1); an accumulate-only step never
+// decays, and only bf16 has a Kahan branch.
+template <template <class, bool, bool, int> class OpT, int NWD, class Fn>
+void dispatch(int dtype, bool kahan, bool update, int wd, Fn&& fn) {
+  auto pick_wd = [&](auto dt, auto kh) {
+    using DT = decltype(dt);
+    constexpr bool K = decltype(kh)::value;
+    if (wd == 1) fn(OpT<DT, K, true, 1>{});
+    else if (wd == 2 && NWD > 2) fn(OpT<DT, K, true, (NWD > 2 ? 2 : 0)>{});
+    else fn(OpT<DT, K, true, 0>{});
+  };
   if (dtype == OPTIMI_BF16) {
-    if (update) {
-      if (kahan) fn(OpT<BF16, true, true>{});
-      else fn(OpT<BF16, false, true>{});
-    } else {
-      fn(OpT<BF16, false, false>{});
-    }
+    if (!update) fn(OpT<BF16, false, false, 0>{});
+    else if (kahan) pick_wd(BF16{}, std::true_type{});
+    else pick_wd(BF16{}, std::false_type{});
   } else {
-    if (update) fn(OpT<F32, false, true>{});
-    else fn(OpT<F32, false, false>{});
+    if (!update) fn(OpT<F32, false, false, 0>{});
+    else pick_wd(F32{}, std::false_type{});
   }
 }
 
 int single_entry(TensorEntry& e, const void* const* ptrs, int n_arrays, uint32_t need, int64_t numel, int dtype) {
   if (numel < 0) return OPTIMI_ERR_SIZE;
   if (dtype != OPTIMI_F32 && dtype != OPTIMI_BF16) return OPTIMI_ERR_DTYPE;
-  if (numel > chunk_elems_rt(dtype) * (int64_t)0x7fffffff) return OPTIMI_ERR_SIZE;
+  if (numel > chunk_elems_rt(dtype) * ((int64_t)0x7fffffff / kSub)) return OPTIMI_ERR_SIZE;
   std::memset(&e, 0, sizeof(e));
   e.numel = numel;
   e.vec_ok = 1;
@@ -759,7 +832,7 @@ int single_entry(TensorEntry& e, const void* const* ptrs, int n_arrays, uint32_t
 
 // ---- scalar packs ------------------------------------------------------------------
 AdamScalars adam_scalars(int dtype, double lr, double beta1_comp, double beta2_hat, double beta2_comp,
-                         double weight_decay, double eps, uint32_t flags) {
+                         double weight_decay, double eps) {
   AdamScalars s;
   s.l1 = make_lerp(beta1_comp);
   s.wd = S(weight_decay);
@@ -768,28 +841,30 @@ AdamScalars adam_scalars(int dtype, double lr, double beta1_comp, double beta2_h
   s.b2c = S(beta2_comp);
   s.eps_d = Sd(eps, dtype);
   s.neg_lr = S(-lr);
-  s.wd_mode = (weight_decay != 0 && (flags & OPTIMI_UPDATE)) ? ((flags & OPTIMI_DECOUPLE_WD) ? 1u : 2u) : 0u;
   return s;
+}
+int adam_wd_mode(double weight_decay, uint32_t flags) {
+  return (weight_decay != 0 && (flags & OPTIMI_UPDATE)) ? ((flags & OPTIMI_DECOUPLE_WD) ? 1 : 2) : 0;
 }
 uint32_t adam_need(bool kahan, bool update) {
   return update ? (bit(0) | bit(1) | bit(2) | bit(3) | (kahan ? bit(4) : 0)) : (bit(1) | bit(2) | bit(3));
 }
 
-LionScalars lion_scalars(int dtype, double lr, double beta1_comp, double beta2_comp, double weight_decay, uint32_t flags) {
+LionScalars lion_scalars(int dtype, double lr, double beta1_comp, double beta2_comp, double weight_decay) {
   LionScalars s;
   s.l1 = make_lerp(beta1_comp);
   s.l2 = make_lerp(beta2_comp);
   s.wd = S(weight_decay);
   s.neg_lr_d = Sd(-lr, dtype);
-  s.do_wd = (weight_decay != 0 && (flags & OPTIMI_UPDATE)) ? 1u : 0u;
   return s;
 }
+int lion_wd_mode(double weight_decay, uint32_t flags) { return (weight_decay != 0 && (flags & OPTIMI_UPDATE)) ? 1 : 0; }
 uint32_t lion_need(bool kahan, bool update) {
   return update ? (bit(0) | bit(1) | bit(2) | (kahan ? bit(3) : 0)) : (bit(1) | bit(2));
 }
 
 AdanScalars adan_scalars(int dtype, double lr, double beta1_comp, double beta2, double beta2_comp, double beta3_hat,
-                         double beta3_comp, double eps, double weight_decay, uint32_t flags) {
+                         double beta3_comp, double eps, double weight_decay) {
   AdanScalars s;
   s.l1 = make_lerp(beta1_comp);
   s.l2 = make_lerp(beta2_comp);
@@ -800,8 +875,10 @@ AdanScalars adan_scalars(int dtype, double lr, double beta1_comp, double beta2, 
   s.neg_lr = S(-lr);
   s.neg_lr_b2 = S(-lr * beta2);
   s.wd = S(weight_decay);
-  s.wd_mode = (weight_decay != 0 && (flags & OPTIMI_UPDATE)) ? ((flags & OPTIMI_ADAM_WD) ? 1u : 2u) : 0u;
   return s;
+}
+int adan_wd_mode(double weight_decay, uint32_t flags) {
+  return (weight_decay != 0 && (flags & OPTIMI_UPDATE)) ? ((flags & OPTIMI_ADAM_WD) ? 1 : 2) : 0;
 }
 uint32_t adan_need(bool kahan, bool update) {
   return bit(1) | bit(2) | bit(3) | bit(4) | bit(5) | (update ? (bit(0) | (kahan ? bit(6) : 0)) : 0);
@@ -835,7 +912,7 @@ int stable_run(bool multi, optimi_group* g, const TensorEntry& single, int n_ten
     else launch_single<StablePass1Op<DT, false>>(single, s1, nullptr, stream);
     return 0;
   }
-  int rc = g->partials.reserve(sizeof(double) * (size_t)n_chunks);
+  int rc = g->partials.reserve(sizeof(double) * (size_t)n_chunks * kSub);
   if (rc) return rc;
   rc = g->tensor_scalars.reserve(sizeof(TensorScalars) * (size_t)(multi ? n_tensors : 1));
   if (rc) return rc;
@@ -849,21 +926,25 @@ int stable_run(bool multi, optimi_group* g, const TensorEntry& single, int n_ten
   s2.eps_d = Sd(eps, dtype);
   s2.neg_lr = 0.0f;
   s2.wd = 0.0f;
-  s2.do_wd = weight_decay != 0 ? 1u : 0u;
+  const bool wd = weight_decay != 0;
   if (multi) {
     launch_multi<StablePass1Op<DT, true>>(g, s1, stream);
     TensorEntry none;
     std::memset(&none, 0, sizeof(none));
-    stable_finalize_kernel<DT, true><<<dim3((unsigned)n_tensors), dim3(kThreads), 0, stream>>>(
+    stable_finalize_kernel<DT, true><<<dim3((unsigned)n_tensors), dim3(kReduceThreads), 0, stream>>>(
         (const TensorEntry*)g->table.ptr, none, (const double*)g->partials.ptr, (TensorScalars*)g->tensor_scalars.ptr, fa);
-    if (kahan) launch_multi<StablePass2Op<DT, true>>(g, s2, stream);
-    else launch_multi<StablePass2Op<DT, false>>(g, s2, stream);
+    if (kahan && wd) launch_multi<StablePass2Op<DT, true, 1>>(g, s2, stream);
+    else if (kahan) launch_multi<StablePass2Op<DT, true, 0>>(g, s2, stream);
+    else if (wd) launch_multi<StablePass2Op<DT, false, 1>>(g, s2, stream);
+    else launch_multi<StablePass2Op<DT, false, 0>>(g, s2, stream);
   } else {
     launch_single<StablePass1Op<DT, true>>(single, s1, (double*)g->partials.ptr, stream);
-    stable_finalize_kernel<DT, false><<<dim3(1), dim3(kThreads), 0, stream>>>(
+    stable_finalize_kernel<DT, false><<<dim3(1), dim3(kReduceThreads), 0, stream>>>(
         nullptr, single, (const double*)g->partials.ptr, (TensorScalars*)g->tensor_scalars.ptr, fa);
-    if (kahan) launch_single<StablePass2Op<DT, true>>(single, s2, nullptr, stream);
-    else launch_single<StablePass2Op<DT, false>>(single, s2, nullptr, stream);
+    if (kahan && wd) launch_single<StablePass2Op<DT, true, 1>>(single, s2, nullptr, stream);
+    else if (kahan) launch_single<StablePass2Op<DT, true, 0>>(single, s2, nullptr, stream);
+    else if (wd) launch_single<StablePass2Op<DT, false, 1>>(single, s2, nullptr, stream);
+    else launch_single<StablePass2Op<DT, false, 0>>(single, s2, nullptr, stream);
   }
   return 0;
 }
@@ -942,8 +1023,8 @@ int optimi_hip_adam_multi(optimi_group* g, int n_tensors, void* const* param, co
   int rc = prepare_tables(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, stream);
   if (rc) return rc;
   if (g->n_chunks == 0) return 0;
-  AdamScalars s = adam_scalars(dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, flags);
-  dispatch3<AdamOp>(dtype, kahan, update, [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
+  AdamScalars s = adam_scalars(dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  dispatch<AdamOp, 3>(dtype, kahan, update, adam_wd_mode(weight_decay, flags), [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
   return note_launch(g, stream);
 }
 
@@ -958,8 +1039,8 @@ int optimi_hip_lion_multi(optimi_group* g, int n_tensors, void* const* param, co
   int rc = prepare_tables(g, n_tensors, lists, 4, lion_need(kahan, update), numel, dtype, stream);
   if (rc) return rc;
   if (g->n_chunks == 0) return 0;
-  LionScalars s = lion_scalars(dtype, lr, beta1_comp, beta2_comp, weight_decay, flags);
-  dispatch3<LionOp>(dtype, kahan, update, [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
+  LionScalars s = lion_scalars(dtype, lr, beta1_comp, beta2_comp, weight_decay);
+  dispatch<LionOp, 2>(dtype, kahan, update, lion_wd_mode(weight_decay, flags), [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
   return note_launch(g, stream);
 }
 
@@ -998,8 +1079,8 @@ int optimi_hip_adan_multi(optimi_group* g, int n_tensors, void* const* param, co
   int rc = prepare_tables(g, n_tensors, lists, 7, adan_need(kahan, update), numel, dtype, stream);
   if (rc) return rc;
   if (g->n_chunks == 0) return 0;
-  AdanScalars s = adan_scalars(dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay, flags);
-  dispatch3<AdanOp>(dtype, kahan, update, [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
+  AdanScalars s = adan_scalars(dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay);
+  dispatch<AdanOp, 3>(dtype, kahan, update, adan_wd_mode(weight_decay, flags), [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
   return note_launch(g, stream);
 }
 
@@ -1013,8 +1094,8 @@ int optimi_hip_adam_single(void* param, const void* grad, void* exp_avg, void* e
   int rc = single_entry(e, ptrs, 5, adam_need(kahan, update), numel, dtype);
   if (rc) return rc;
   if (numel == 0) return 0;
-  AdamScalars s = adam_scalars(dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, flags);
-  dispatch3<AdamOp>(dtype, kahan, update, [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
+  AdamScalars s = adam_scalars(dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  dispatch<AdamOp, 3>(dtype, kahan, update, adam_wd_mode(weight_decay, flags), [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
   HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -1029,8 +1110,8 @@ int optimi_hip_lion_single(void* param, const void* grad, void* exp_avg, void* k
   int rc = single_entry(e, ptrs, 4, lion_need(kahan, update), numel, dtype);
   if (rc) return rc;
   if (numel == 0) return 0;
-  LionScalars s = lion_scalars(dtype, lr, beta1_comp, beta2_comp, weight_decay, flags);
-  dispatch3<LionOp>(dtype, kahan, update, [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
+  LionScalars s = lion_scalars(dtype, lr, beta1_comp, beta2_comp, weight_decay);
+  dispatch<LionOp, 2>(dtype, kahan, update, lion_wd_mode(weight_decay, flags), [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
   HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -1070,8 +1151,8 @@ int optimi_hip_adan_single(void* param, const void* grad, void* exp_avg, void* e
   int rc = single_entry(e, ptrs, 7, adan_need(kahan, update), numel, dtype);
   if (rc) return rc;
   if (numel == 0) return 0;
-  AdanScalars s = adan_scalars(dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay, flags);
-  dispatch3<AdanOp>(dtype, kahan, update, [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
+  AdanScalars s = adan_scalars(dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay);
+  dispatch<AdanOp, 3>(dtype, kahan, update, adan_wd_mode(weight_decay, flags), [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
   HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -1082,10 +1163,9 @@ int optimi_hip_copy_probe(void* dst, const void* src, int64_t bytes, optimi_stre
   if (((uintptr_t)dst % 16) || ((uintptr_t)src % 16)) return OPTIMI_ERR_ALIGN;
   const int64_t n_vec = bytes / 16;
   if (n_vec == 0) return 0;
-  const int64_t per_block = (int64_t)kThreads * kUnroll;
-  const int64_t blocks = (n_vec + per_block - 1) / per_block;
+  const int64_t blocks = (n_vec + 255) / 256;
   if (blocks > 0x7fffffff) return OPTIMI_ERR_SIZE;
-  copy_probe_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream_>>>((u32x4*)dst, (const u32x4*)src, n_vec);
+  copy_probe_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream_>>>((u32x4*)dst, (const u32x4*)src, n_vec);
   HIP_TRY(hipGetLastError());
   return 0;
 }
