@@ -7,8 +7,8 @@
 // stands where the reference enters its Triton launchers (optimi/adam.py:278-291,
 // lion.py:240-253, stableadamw.py:337-350, adan.py:314-327).
 
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
 #include <cmath>
@@ -126,10 +126,10 @@ void adam_multi(Group& group, const TensorList& params, const TensorList& grads,
   Prepared pr = prepare(params, flags);
   PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
   PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
-  c10::hip::HIPGuard guard(params[0].device());
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
   check_status(optimi_hip_adam_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
                                      pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp, beta2_hat,
-                                     beta2_comp, weight_decay, eps, flags, c10::hip::getCurrentHIPStream().stream()),
+                                     beta2_comp, weight_decay, eps, flags, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
                "optimi_hip_adam_multi");
 }
 
@@ -140,10 +140,10 @@ void lion_multi(Group& group, const TensorList& params, const TensorList& grads,
   Prepared pr = prepare(params, flags);
   PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg");
   PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
-  c10::hip::HIPGuard guard(params[0].device());
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
   check_status(optimi_hip_lion_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(),
                                      pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp, beta2_comp,
-                                     weight_decay, flags, c10::hip::getCurrentHIPStream().stream()),
+                                     weight_decay, flags, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
                "optimi_hip_lion_multi");
 }
 
@@ -155,11 +155,11 @@ void stableadamw_multi(Group& group, const TensorList& params, const TensorList&
   Prepared pr = prepare(params, flags);
   PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
   PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
-  c10::hip::HIPGuard guard(params[0].device());
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
   check_status(optimi_hip_stableadamw_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
                                             pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp,
                                             beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags,
-                                            c10::hip::getCurrentHIPStream().stream()),
+                                            c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
                "optimi_hip_stableadamw_multi");
 }
 
@@ -173,11 +173,11 @@ void adan_multi(Group& group, const TensorList& params, const TensorList& grads,
   PtrList df = gather(params, exp_avg_diffs, "exp_avg_diff"), n = gather(params, exp_avg_sqs, "exp_avg_sq");
   PtrList pg = gather(params, prev_grads, "prev_grad");
   PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
-  c10::hip::HIPGuard guard(params[0].device());
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
   check_status(optimi_hip_adan_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), df.data(),
                                      n.data(), pg.data(), pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr,
                                      beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay, flags,
-                                     c10::hip::getCurrentHIPStream().stream()),
+                                     c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
                "optimi_hip_adan_multi");
 }
 
@@ -208,10 +208,10 @@ void adam_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, 
   check_like(p, g, "grad");
   check_like(p, m, "exp_avg");
   check_like(p, v, "exp_avg_sq");
-  c10::hip::HIPGuard guard(p.device());
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(p.device());
   check_status(optimi_hip_adam_single(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), o.k, p.numel(), o.dtype, lr,
                                       beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, flags,
-                                      c10::hip::getCurrentHIPStream().stream()),
+                                      c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
                "optimi_hip_adam_single");
 }
 
@@ -220,9 +220,9 @@ void lion_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, 
   One o = prepare_one(p, kahan_comp, flags);
   check_like(p, g, "grad");
   check_like(p, m, "exp_avg");
-  c10::hip::HIPGuard guard(p.device());
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(p.device());
   check_status(optimi_hip_lion_single(p.data_ptr(), g.data_ptr(), m.data_ptr(), o.k, p.numel(), o.dtype, lr, beta1_comp,
-                                      beta2_comp, weight_decay, flags, c10::hip::getCurrentHIPStream().stream()),
+                                      beta2_comp, weight_decay, flags, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
                "optimi_hip_lion_single");
 }
 
@@ -233,10 +233,10 @@ void stableadamw_single(Group& group, const at::Tensor& p, const at::Tensor& g, 
   check_like(p, g, "grad");
   check_like(p, m, "exp_avg");
   check_like(p, v, "exp_avg_sq");
-  c10::hip::HIPGuard guard(p.device());
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(p.device());
   check_status(optimi_hip_stableadamw_single(group.get(), p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), o.k,
                                              p.numel(), o.dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps,
-                                             max_lr, flags, c10::hip::getCurrentHIPStream().stream()),
+                                             max_lr, flags, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
                "optimi_hip_stableadamw_single");
 }
 
@@ -250,10 +250,10 @@ void adan_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, 
   check_like(p, df, "exp_avg_diff");
   check_like(p, n, "exp_avg_sq");
   check_like(p, pg, "prev_grad");
-  c10::hip::HIPGuard guard(p.device());
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(p.device());
   check_status(optimi_hip_adan_single(p.data_ptr(), g.data_ptr(), m.data_ptr(), df.data_ptr(), n.data_ptr(), pg.data_ptr(),
                                       o.k, p.numel(), o.dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp,
-                                      eps, weight_decay, flags, c10::hip::getCurrentHIPStream().stream()),
+                                      eps, weight_decay, flags, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
                "optimi_hip_adan_single");
 }
 

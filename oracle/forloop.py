@@ -262,11 +262,21 @@ class ForLoopRun:
     and one step counter per group or – in gradient-release mode – per tensor.
     """
 
+    # constructor defaults of the reference classes (adam.py:56-70, adamw.py:48-61, lion.py:56-68,
+    # stableadamw.py:76-89, adan.py:62-76); ``lr`` is always required
+    DEFAULTS = {
+        "adam": dict(betas=(0.9, 0.99), weight_decay=0.0, eps=1e-6, decouple_wd=False),
+        "adamw": dict(betas=(0.9, 0.99), weight_decay=1e-2, eps=1e-6),
+        "lion": dict(betas=(0.9, 0.99), weight_decay=0.0),
+        "stableadamw": dict(betas=(0.9, 0.99), weight_decay=1e-2, eps=1e-6),
+        "adan": dict(betas=(0.98, 0.92, 0.99), weight_decay=2e-2, eps=1e-6),
+    }
+
     def __init__(self, name, params, *, gradient_release=False, **hyper):
         self.name = name
         self.params = list(params)
         self.gradient_release = gradient_release
-        self.hyper = dict(hyper)
+        self.hyper = {**self.DEFAULTS[name], **hyper}
         if self.hyper.get("decouple_lr") and self.hyper.get("max_lr") is None:
             self.hyper["max_lr"] = self.hyper["lr"]  # optimizer.py:20-21
         ks = self.hyper.pop("kahan_sum", False if name == "adan" else None)

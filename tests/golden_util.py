@@ -100,3 +100,57 @@ def fp32_rel_err(a: torch.Tensor, b: torch.Tensor, floor: float) -> torch.Tensor
     """|a-b| / max(|a|,|b|, floor)."""
     a, b = a.double(), b.double()
     return (a - b).abs() / torch.maximum(torch.maximum(a.abs(), b.abs()), torch.tensor(floor, dtype=torch.float64))
+
+
+def assert_bits_equal(got: torch.Tensor, want: torch.Tensor, what: str):
+    a = got.detach().cpu().contiguous()
+    b = want.detach().cpu().contiguous()
+    view = torch.int16 if a.dtype == torch.bfloat16 else torch.int32
+    bad = a.view(view) != b.view(view)
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} elements differ (first at {int(bad.flatten().nonzero()[0])})"
+
+
+def assert_close_to_reference(got, want, what, *, param=None, is_param=False):
+    """The north-star tolerance: bf16 within 1 ulp (a Kahan buffer within 1 ulp of its parameter),
+    fp32 within rel 1e-6.  The fp32 comparison is |a-b| <= 1e-6 * max(|a|, |b|, floor): elements
+    that cancel towards zero carry the rounding error of the terms that cancelled, so they are
+    judged against the size of those terms - 1e-2 for parameters (the distance ten steps can move
+    a parameter at lr 1e-3; i.e. |a-b| <= 1e-8 near zero) and the tensor's RMS for moment states."""
+    got, want = got.detach().cpu(), want.detach().cpu()
+    if want.dtype == torch.bfloat16:
+        if param is not None:
+            err = (got.float() - want.float()).abs() / bf16_ulp_of(param.detach().cpu())
+            assert float(err.max()) <= 1.0, f"{what}: Kahan buffer off by {float(err.max()):.3f} parameter ulps"
+        else:
+            ulp = bf16_ulp_diff(got, want)
+            assert int(ulp.max()) <= 1, f"{what}: {int((ulp > 1).sum())} elements beyond 1 ulp (max {int(ulp.max())})"
+    else:
+        floor = 1e-2 if is_param else max(float(want.double().pow(2).mean().sqrt()), 1e-30)
+        rel = fp32_rel_err(got, want, floor)
+        assert float(rel.max()) <= 1e-6, f"{what}: rel err {float(rel.max()):.3e}"
+
+
+def compare_engines(got_eng, want_eng, what, exact: bool, body_only: int = 0):
+    """Params and every state of two engines; ``exact`` demands bit equality.  ``body_only=w``
+    leaves out the last ``numel % w`` elements of every tensor (the part a CPU kernel of vector
+    width ``w`` handles in its scalar remainder loop)."""
+    for i, (p, q) in enumerate(zip(got_eng.params, want_eng.params)):
+        keep = p.numel() - (p.numel() % body_only if body_only else 0)
+        if keep == 0:
+            continue
+        items = [("param", p, q)]
+        for key in STATE_KEYS:
+            a = got_eng.state[i].get(key) if got_eng.state[i] else None
+            b = want_eng.state[i].get(key) if want_eng.state[i] else None
+            assert (a is None) == (b is None), f"{what} tensor {i} {key}: present in one engine only"
+            if a is not None:
+                items.append((key, a, b))
+        for key, a, b in items:
+            label = f"{what} tensor {i} ({tuple(p.shape)}) {key}"
+            a, b = a.detach().flatten()[:keep], b.detach().flatten()[:keep]
+            if key == "kahan_comp":
+                q = q.detach().flatten()[:keep]
+            if exact:
+                assert_bits_equal(a, b, label)
+            else:
+                assert_close_to_reference(a, b, label, param=q if key == "kahan_comp" else None, is_param=key == "param")

@@ -1,0 +1,47 @@
+"""Both oracles against the golden vectors written by the reference (tests/golden/*.npz).
+
+* ``oracle.forloop.ForLoopRun`` (same torch ops, same order) must reproduce every snapshot
+  bit for bit: it runs the reference's arithmetic on the reference's inputs.
+* ``oracle.scalar.ScalarRun`` (hand-written rounding points in C) must be bit-exact on bf16
+  tensors and on fp32 moment states.  fp32 parameters may differ in the last bits because
+  torch's CPU sqrt is faithfully, not correctly, rounded, and StableAdamW's mean is summed in
+  another order: there the bar is |a-b| <= 1e-6 * max(|a|, |b|, 1e-3).
+"""
+
+import pytest
+import torch
+
+import golden_util as G
+from oracle.forloop import ForLoopRun
+from oracle.scalar import ScalarRun
+
+
+def bits(t):
+    return t.contiguous().view(torch.int16 if t.dtype == torch.bfloat16 else torch.int32)
+
+
+@pytest.mark.parametrize("name", G.case_names())
+def test_forloop_restatement_is_bit_exact(name):
+    torch.set_num_threads(1)
+    fx = G.load(name)
+    out = G.replay(name, fx, ForLoopRun)
+    wanted = sorted(k for k in fx if k.startswith("out."))
+    assert sorted(out) == wanted
+    for k in wanted:
+        assert torch.equal(bits(out[k]), bits(fx[k])), f"{name} {k}"
+
+
+@pytest.mark.parametrize("name", G.case_names())
+def test_scalar_emulator(name):
+    fx = G.load(name)
+    out = G.replay(name, fx, ScalarRun)
+    wanted = sorted(k for k in fx if k.startswith("out."))
+    assert sorted(out) == wanted
+    for k in wanted:
+        got, want = out[k], fx[k]
+        if want.dtype == torch.bfloat16 or ".param." not in k:
+            n_bad = int((bits(got) != bits(want)).sum())
+            assert n_bad == 0, f"{name} {k}: {n_bad} elements differ"
+        else:
+            rel = G.fp32_rel_err(got, want, 1e-3)
+            assert float(rel.max()) <= 1e-6, f"{name} {k}: rel err {float(rel.max())}"
