@@ -59,7 +59,10 @@ def workloads():
 
 # HBM bytes per step read off the hardware counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for a plain copy of known size).  None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/adamw_bf16_kahan_llama7b_hbm_traffic.txt: 67.44 GB read + 53.90 GB written
+    "adamw_bf16_kahan_llama7b": 1.2134e11,
+}
 
 
 def numel(shape):
@@ -127,6 +130,9 @@ def main():
     ap.add_argument("--workload", default="adamw_bf16_kahan_llama7b")
     ap.add_argument("--grad-sets", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe-bytes", type=int, default=0,
+                    help="also run the library's plain copy kernel over this many bytes (3 launches) before the "
+                         "workload; a profiler run uses it to scale its byte counters against a known size")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -140,6 +146,17 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no HIP device visible")
     device = torch.device("cuda:0")
+    if args.copy_probe_bytes:
+        from optimi_amd import cabi
+
+        n = args.copy_probe_bytes // 16 * 16
+        src = torch.zeros(n, dtype=torch.uint8, device=device)
+        dst = torch.ones(n, dtype=torch.uint8, device=device)
+        for _ in range(3):
+            cabi.check(cabi.lib().optimi_hip_copy_probe(dst.data_ptr(), src.data_ptr(), n, torch.cuda.current_stream().cuda_stream),
+                       "optimi_hip_copy_probe")
+        torch.cuda.synchronize()
+        del src, dst
     cls_name, kwargs, dtype_name, shapes, bytes_per_param = workloads()[args.workload]
     dtype = getattr(torch, dtype_name)
     n_params = sum(numel(s) for s in shapes)

@@ -67,13 +67,8 @@ __device__ __forceinline__ void store16(void* base, int64_t byte_off, u32x4 v) {
 // rounds two values.  With packed fp32 ops disabled the pair arithmetic is two scalar ops.
 __device__ __forceinline__ f32x2 splat(float x) { return f32x2{x, x}; }
 __device__ __forceinline__ f32x2 fma2(f32x2 a, f32x2 b, f32x2 c) { return f32x2{fmaf(a.x, b.x, c.x), fmaf(a.y, b.y, c.y)}; }
-#ifdef OPTIMI_PROBE_FAST  // measurement only: how much the exact sqrt/divide sequences cost
-__device__ __forceinline__ f32x2 sqrt2(f32x2 a) { return f32x2{__builtin_amdgcn_sqrtf(a.x), __builtin_amdgcn_sqrtf(a.y)}; }
-__device__ __forceinline__ f32x2 div2(f32x2 a, f32x2 b) { return f32x2{a.x * __builtin_amdgcn_rcpf(b.x), a.y * __builtin_amdgcn_rcpf(b.y)}; }
-#else
 __device__ __forceinline__ f32x2 sqrt2(f32x2 a) { return f32x2{sqrtf(a.x), sqrtf(a.y)}; }
 __device__ __forceinline__ f32x2 div2(f32x2 a, f32x2 b) { return f32x2{a.x / b.x, a.y / b.y}; }
-#endif
 
 // ------------------------------------------------------------------------------------
 // dtype policies
