@@ -1,0 +1,173 @@
+"""Parity at the sizes of the BASELINE configurations.
+
+* C2 – AdamW bf16 + Kahan, ``decouple_lr``, wd 1e-5, the whole Llama-1B-shaped list (147 tensors,
+  1,204,881,408 params), 10 steps with fresh gradients: every tensor against the C emulator, bit-exact.
+* C3/C4 – Lion, StableAdamW, Adan in bf16 + Kahan on the Llama-7B-shaped list (290 tensors,
+  6,738,411,520 params): the whole list is stepped in one launch, and a sample of tensors that
+  covers all five distinct shapes is also stepped through the per-tensor entry point from cloned
+  inputs – a whole-list launch must equal per-tensor launches bit for bit, whatever the list size.
+  The same sample is checked against the C emulator on the CPU (10 steps).
+* C5 – AdamW bf16 + Kahan per tensor in reverse order with ``accumulation_steps=4`` on the 7B shapes
+  sample, and the 10,000-tensor stress list (sizes log-uniform in [128, 65536]) both as one launch and
+  as 10,000 per-tensor launches, against the C emulator.
+Gradients are drawn on the GPU (seeded) and copied to the host for the oracle.
+"""
+
+import math
+
+import pytest
+import torch
+
+import golden_util as G
+from oracle.scalar import ScalarRun
+
+pytestmark = pytest.mark.gpu
+
+ADAMW = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
+HYPER = {
+    "lion": dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1),
+    "stableadamw": dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2),
+    "adan": dict(lr=1e-3, betas=(0.98, 0.92, 0.99), eps=1e-8, weight_decay=2e-2, kahan_sum=True),
+    "adamw": ADAMW,
+}
+
+
+def llama_shapes(hidden, inter, layers, vocab=32000, final_norm=False):
+    shapes = [(vocab, hidden)]
+    for _ in range(layers):
+        shapes += [(hidden, hidden)] * 4 + [(inter, hidden)] * 2 + [(hidden, inter)] + [(hidden,)] * 2
+    if final_norm:
+        shapes.append((hidden,))
+    shapes.append((vocab, hidden))
+    return shapes
+
+
+def draw(shapes, device, gen, std, ones_for_1d=False):
+    out = []
+    for s in shapes:
+        if ones_for_1d and len(s) == 1:
+            out.append(torch.ones(s, dtype=torch.bfloat16, device=device))
+        else:
+            out.append(torch.empty(s, dtype=torch.float32, device=device).normal_(0, std, generator=gen).bfloat16())
+    return out
+
+
+def free():
+    import gc
+
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def test_c2_adamw_llama1b_whole_list(hip_device):
+    from hip_engine import HipRun
+
+    shapes = llama_shapes(2048, 8192, 16, final_norm=True)
+    assert len(shapes) == 147 and sum(math.prod(s) for s in shapes) == 1_204_881_408
+    hyper = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-5, decouple_lr=True)
+    gen = torch.Generator(device=hip_device).manual_seed(2)
+    params = draw(shapes, hip_device, gen, 0.02, ones_for_1d=True)
+    hip = HipRun("adamw", params, **hyper)
+    sca = ScalarRun("adamw", [p.cpu() for p in params], **hyper)
+    for _ in range(10):
+        grads = draw(shapes, hip_device, gen, 1e-3)
+        hip.step(grads)
+        sca.step([g.cpu() for g in grads])
+        del grads
+    G.compare_engines(hip, sca, "C2", exact=True)
+    del hip, sca, params
+    free()
+
+
+SAMPLE_7B = [0, 1, 5, 6, 7, 8, 9, 143, 147, 280, 288, 289]  # embed, q, gate, up, down, both norms, ..., lm_head
+
+
+@pytest.mark.parametrize("name", ["lion", "stableadamw", "adan", "adamw"])
+def test_c3_c4_llama7b_whole_list_equals_per_tensor(name, hip_device):
+    from hip_engine import HipRun
+
+    shapes = llama_shapes(4096, 11008, 32)
+    assert len(shapes) == 290 and sum(math.prod(s) for s in shapes) == 6_738_411_520
+    hyper = HYPER[name]
+    gen = torch.Generator(device=hip_device).manual_seed(3)
+    params = draw(shapes, hip_device, gen, 0.02, ones_for_1d=True)
+    sample = HipRun(name, [params[i].clone() for i in SAMPLE_7B], gradient_release=True, **hyper)  # per-tensor entry points
+    whole = HipRun(name, params, **hyper)
+    for _ in range(2):
+        grads = draw(shapes, hip_device, gen, 1e-3)
+        for j, i in enumerate(SAMPLE_7B):
+            sample.step_param(j, grads[i].clone())
+        whole.step(grads)
+        del grads
+    torch.cuda.synchronize()
+    for j, i in enumerate(SAMPLE_7B):
+        G.assert_bits_equal(whole.params[i], sample.params[j], f"{name} tensor {i} param")
+        for key in G.STATE_KEYS:
+            a = whole.state[i].get(key)
+            if a is not None:
+                G.assert_bits_equal(a, sample.state[j][key], f"{name} tensor {i} {key}")
+    del whole, sample, params
+    free()
+
+
+DISTINCT_7B = [(32000, 4096), (4096, 4096), (11008, 4096), (4096, 11008), (4096,)]
+
+
+@pytest.mark.parametrize("name", ["lion", "stableadamw", "adan"])
+def test_c3_c4_distinct_7b_shapes_against_emulator(name, hip_device):
+    from hip_engine import HipRun
+
+    hyper = HYPER[name]
+    gen = torch.Generator(device=hip_device).manual_seed(4)
+    params = draw(DISTINCT_7B, hip_device, gen, 0.02, ones_for_1d=True)
+    hip = HipRun(name, params, **hyper)
+    sca = ScalarRun(name, [p.cpu() for p in params], **hyper)
+    for _ in range(10):
+        grads = draw(DISTINCT_7B, hip_device, gen, 1e-3)
+        hip.step(grads)
+        sca.step([g.cpu() for g in grads])
+    G.compare_engines(hip, sca, f"{name} 7B shapes", exact=name != "stableadamw")
+    del hip, sca, params
+    free()
+
+
+def test_c5_release_with_accumulation_7b_shapes(hip_device):
+    from hip_engine import HipRun
+
+    gen = torch.Generator(device=hip_device).manual_seed(5)
+    params = draw(DISTINCT_7B, hip_device, gen, 0.02, ones_for_1d=True)
+    hip = HipRun("adamw", params, gradient_release=True, **ADAMW)
+    sca = ScalarRun("adamw", [p.cpu() for p in params], gradient_release=True, **ADAMW)
+    for t in range(8):
+        hip.optimizer_accumulation = sca.optimizer_accumulation = (t + 1) % 4 != 0
+        grads = draw(DISTINCT_7B, hip_device, gen, 1e-3)
+        for i in reversed(range(len(params))):
+            hip.step_param(i, grads[i])
+            sca.step_param(i, grads[i].cpu())
+    G.compare_engines(hip, sca, "C5 release", exact=True)
+    del hip, sca, params
+    free()
+
+
+def test_c5_stress_list_10000_tensors(hip_device):
+    from hip_engine import HipRun
+
+    rng = torch.Generator().manual_seed(6)
+    sizes = torch.exp(torch.empty(10_000).uniform_(math.log(128), math.log(65536), generator=rng)).long().clamp(128, 65536).tolist()
+    assert len(sizes) == 10_000 and 0.8e8 < sum(sizes) < 1.3e8
+    shapes = [(n,) for n in sizes]
+    gen = torch.Generator(device=hip_device).manual_seed(7)
+    params = draw(shapes, hip_device, gen, 0.02)
+    multi = HipRun("adamw", [p.clone() for p in params], **ADAMW)
+    single = HipRun("adamw", [p.clone() for p in params], gradient_release=True, **ADAMW)
+    sca = ScalarRun("adamw", [p.cpu() for p in params], **ADAMW)
+    for _ in range(3):
+        grads = draw(shapes, hip_device, gen, 1e-3)
+        multi.step(grads)
+        for i in reversed(range(len(shapes))):
+            single.step_param(i, grads[i])
+        sca.step([g.cpu() for g in grads])
+    G.compare_engines(multi, sca, "stress multi", exact=True)
+    G.compare_engines(single, multi, "stress per-tensor", exact=True)
+    del multi, single, sca, params
+    free()
