@@ -257,6 +257,88 @@ void adan_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, 
                "optimi_hip_adan_single");
 }
 
+
+// ---- gradient-release fast path --------------------------------------------------------
+// One call per parameter from the post-accumulate-grad hook: advances the parameter's int32
+// CPU step counter, forms the step scalars in double exactly as the functional forms do in
+// Python (optimi/adam.py:260-273, lion.py:226-235, stableadamw.py:326-332, adan.py:289-309)
+// and launches the per-tensor kernel.  std::pow(double, double) is libm's pow, the function
+// CPython's float ** int ends in, so the scalars are bit-identical to the Python path.
+
+double debias_beta(double beta, int64_t step) {  // optimi/utils.py:31-36
+  const double bt = std::pow(beta, (double)step);
+  return (bt - beta) / (bt - 1.0);
+}
+
+int64_t tick(const at::Tensor& step) {
+  TORCH_CHECK(step.device().is_cpu() && step.scalar_type() == at::kInt && step.numel() == 1,
+              "optimi_amd: the step counter must be a one-element int32 CPU tensor");
+  int32_t* s = step.data_ptr<int32_t>();
+  *s += 1;
+  return *s;
+}
+
+// The Kahan buffer if it is one: placeholders (one element, maybe another dtype) and None count as absent.
+std::optional<at::Tensor> real_kahan(const at::Tensor& p, const std::optional<at::Tensor>& k) {
+  if (!k.has_value() || !k->defined() || k->numel() != p.numel() || k->scalar_type() != p.scalar_type()) return std::nullopt;
+  return k;
+}
+
+at::Tensor grad_like(const at::Tensor& p, const at::Tensor& g) {
+  TORCH_CHECK(g.scalar_type() == p.scalar_type(), "optimi_amd: gradient dtype ", g.scalar_type(), " differs from parameter dtype ", p.scalar_type());
+  if (g.strides() == p.strides()) return g;
+  return at::empty_like(p).copy_(g);
+}
+
+uint32_t base_flags(bool kahan_sum, bool update) { return (kahan_sum ? OPTIMI_KAHAN : 0u) | (update ? OPTIMI_UPDATE : 0u); }
+
+void adam_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
+                  const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
+                  double weight_decay, double eps, bool decouple_wd, bool decouple_lr, std::optional<double> max_lr,
+                  bool kahan_sum, bool update) {
+  const int64_t t = tick(step);
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
+  if (weight_decay != 0) {
+    if (decouple_lr) weight_decay = 1 - (lr / max_lr.value()) * weight_decay;
+    else if (decouple_wd) weight_decay = 1 - lr * weight_decay;
+  }
+  const uint32_t flags = base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u);
+  adam_single(p, grad_like(p, g), m, v, real_kahan(p, k), lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps, flags);
+}
+
+void lion_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const std::optional<at::Tensor>& k,
+                  double lr, double beta1, double beta2, double weight_decay, bool decouple_lr,
+                  std::optional<double> max_lr, bool kahan_sum, bool update) {
+  if (weight_decay != 0) weight_decay = decouple_lr ? 1 - (lr / max_lr.value()) * weight_decay : 1 - lr * weight_decay;
+  lion_single(p, grad_like(p, g), m, real_kahan(p, k), lr, 1 - beta1, 1 - beta2, weight_decay, base_flags(kahan_sum, update));
+}
+
+void stableadamw_release(Group& group, const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
+                         const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
+                         double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum,
+                         bool update) {
+  const int64_t t = tick(step);
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
+  const uint32_t flags = base_flags(kahan_sum, update) | (decouple_lr ? OPTIMI_DECOUPLE_LR : 0u);
+  stableadamw_single(group, p, grad_like(p, g), m, v, real_kahan(p, k), lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps,
+                     (decouple_lr && max_lr.has_value()) ? *max_lr : 0.0, flags);
+}
+
+void adan_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& df, const at::Tensor& n,
+                  const at::Tensor& pg, const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1,
+                  double beta2, double beta3, double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr,
+                  bool adam_wd, bool kahan_sum, bool update) {
+  const int64_t t = tick(step);
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t), b3h = debias_beta(beta3, t);
+  if (weight_decay != 0) {
+    weight_decay = decouple_lr ? (lr / max_lr.value()) * weight_decay : lr * weight_decay;
+    weight_decay = adam_wd ? 1 - weight_decay : 1 + weight_decay;
+  }
+  const uint32_t flags = base_flags(kahan_sum, update) | (adam_wd ? OPTIMI_ADAM_WD : 0u);
+  adan_single(p, grad_like(p, g), m, df, n, pg, real_kahan(p, k), lr, 1 - b1h, beta2, 1 - b2h, b3h, 1 - b3h, eps, weight_decay,
+              flags);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
@@ -276,4 +358,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.def("lion_single", &lion_single);
   mod.def("stableadamw_single", &stableadamw_single);
   mod.def("adan_single", &adan_single);
+  mod.def("adam_release", &adam_release);
+  mod.def("lion_release", &lion_release);
+  mod.def("stableadamw_release", &stableadamw_release);
+  mod.def("adan_release", &adan_release);
+  mod.def("debias_beta", &debias_beta);
 }

@@ -15,8 +15,8 @@ __all__ = ["prepare_for_gradient_release", "remove_gradient_release"]
 
 
 def _gradient_release_hook(param: Tensor, optimizer: OptimiOptimizer):
-    optimizer.step(param=param)
-    optimizer.zero_grad(param=param)
+    # step(param=param) then zero_grad(param=param), in one native call per parameter
+    optimizer._release(param)
 
 
 def prepare_for_gradient_release(model: Module, optimizer: OptimiOptimizer, ignore_existing_hooks: bool = False):

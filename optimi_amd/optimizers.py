@@ -18,6 +18,9 @@ import torch
 from torch import Tensor
 from torch.optim.optimizer import Optimizer
 
+from torch.optim import optimizer as _torch_optimizer
+
+from . import backend
 from . import functional as F
 
 __all__ = ["OptimiOptimizer", "Adam", "AdamW", "Lion", "StableAdamW", "Adan"]
@@ -198,6 +201,39 @@ class OptimiOptimizer(Optimizer):
             self._functional(group, param, param.grad, state, state.get("step"), True, self._optimizer_accumulation)
         return loss
 
+    # -- gradient-release fast path --------------------------------------------------------
+    def _release_call(self, ext, group, state, param, grad, update):
+        """One native call that advances the parameter's step counter, forms the step scalars and
+        launches the per-tensor kernel.  Subclasses forward their hyper-parameters."""
+        raise NotImplementedError
+
+    def _has_step_hooks(self) -> bool:
+        return bool(self._optimizer_step_pre_hooks or self._optimizer_step_post_hooks
+                    or _torch_optimizer._global_optimizer_pre_hooks or _torch_optimizer._global_optimizer_post_hooks)
+
+    @torch.no_grad()
+    def _release(self, param: Tensor):
+        """``step(param=param)`` followed by ``zero_grad(param=param)``, as the post-accumulate-grad
+        hook needs it (optimi/gradientrelease.py:13-15), with the scalar prologue done natively.
+        Same results as the public path; it only skips the per-call Python work, which dominates
+        when a model has thousands of small tensors.  Falls back to the public methods when step
+        hooks are registered, so they still fire."""
+        if self._has_step_hooks():
+            self.step(param=param)
+            self.zero_grad(param=param)
+            return
+        state = self.state[param]
+        group = state["group"]
+        if "kahan_comp" not in state:
+            if group["triton"] is None:
+                group["triton"] = _default_to_fused([param])
+            self._init_state(group, state, param, True)
+        if not group["triton"]:
+            raise RuntimeError("optimi_amd: parameter is not eligible for the HIP backend and there is no other backend")
+        backend.check_supported(param)
+        self._release_call(backend.ext(), group, state, param, param.grad, not self._optimizer_accumulation)
+        param.grad = None
+
     @torch._disable_dynamo
     def zero_grad(self, set_to_none: bool = True, param: Tensor | None = None):
         """Resets the gradients of all optimized parameters or individual parameter.
@@ -279,6 +315,12 @@ class Adam(OptimiOptimizer):
                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
 
+    def _release_call(self, ext, group, state, param, grad, update):
+        ext.adam_release(param, grad, state["exp_avg"], state["exp_avg_sq"], state["kahan_comp"], state["step"], group["lr"],
+                         group["beta1"], group["beta2"], group["weight_decay"], group["eps"], group["decouple_wd"],
+                         group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update)
+
+
 class AdamW(Adam):
     """AdamW optimizer: Adam with decoupled weight decay.
 
@@ -349,6 +391,11 @@ class Lion(OptimiOptimizer):
                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
 
+    def _release_call(self, ext, group, state, param, grad, update):
+        ext.lion_release(param, grad, state["exp_avg"], state["kahan_comp"], group["lr"], group["beta1"], group["beta2"],
+                         group["weight_decay"], group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update)
+
+
 def _restore_scratch_state(optim: OptimiOptimizer):
     """``load_state_dict`` casts floating state to the parameter dtype; bring the fp32 scratch
     back (optimi/stableadamw.py:38-47)."""
@@ -417,6 +464,13 @@ class StableAdamW(OptimiOptimizer):
                       _groups=self._hip_groups)
 
 
+    def _release_call(self, ext, group, state, param, grad, update):
+        grp = F._workspace(self._hip_groups, param.device, param.dtype, "stableadamw_single")
+        ext.stableadamw_release(grp, param, grad, state["exp_avg"], state["exp_avg_sq"], state["kahan_comp"], state["step"],
+                                group["lr"], group["beta1"], group["beta2"], group["weight_decay"], group["eps"],
+                                group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update)
+
+
 class Adan(OptimiOptimizer):
     """Adan Optimizer: Adaptive Nesterov Momentum Algorithm.
 
@@ -478,3 +532,10 @@ class Adan(OptimiOptimizer):
                step=step, decouple_lr=group["decouple_lr"], max_lr=group["max_lr"], kahan_sum=group["kahan_sum"],
                foreach=False, triton=True, gradient_release=gradient_release,
                optimizer_accumulation=accumulate, _groups=self._hip_groups)
+
+    def _release_call(self, ext, group, state, param, grad, update):
+        # adam_wd is not forwarded, as in step() above
+        ext.adan_release(param, grad, state["exp_avg"], state["exp_avg_diff"], state["exp_avg_sq"], state["prev_grad"],
+                         state["kahan_comp"], state["step"], group["lr"], group["beta1"], group["beta2"], group["beta3"],
+                         group["weight_decay"], group["eps"], group["decouple_lr"], group["max_lr"], False,
+                         bool(group["kahan_sum"]), update)

@@ -168,3 +168,47 @@ def test_noncontiguous_gradient_is_relaid(hip_device):
     opt.step()
     ref.step([g.cpu().contiguous()])
     G.assert_close_to_reference(p, ref.params[0], "strided grad", is_param=True)
+
+
+@pytest.mark.parametrize("case", ["adamw", "adamw_declr", "lion", "stableadamw", "adan"])
+def test_release_fast_path_equals_public_step(case, hip_device):
+    """The hook's one-call native path and ``step(param=p); zero_grad(param=p)`` give the same bits,
+    including the accumulate-only micro-steps and the per-parameter step counters."""
+    cls, _, hyper = CASES[case]
+    torch.manual_seed(0)
+    p0 = [(torch.randn(s) * 0.02).bfloat16().to(hip_device) for s in [(300, 70), (8200,), (5,)]]
+    a = [torch.nn.Parameter(p.clone()) for p in p0]
+    b = [torch.nn.Parameter(p.clone()) for p in p0]
+    fast, public = cls(a, gradient_release=True, **hyper), cls(b, gradient_release=True, **hyper)
+    gen = torch.Generator().manual_seed(9)
+    for it in range(8):
+        fast.optimizer_accumulation = public.optimizer_accumulation = (it + 1) % 4 != 0
+        for pa, pb in zip(reversed(a), reversed(b)):
+            g = (torch.randn(pa.shape, generator=gen) * 1e-3).bfloat16().to(hip_device)
+            pa.grad, pb.grad = g.clone(), g.clone()
+            fast._release(pa)
+            public.step(param=pb)
+            public.zero_grad(param=pb)
+            assert pa.grad is None and pb.grad is None
+    for pa, pb in zip(a, b):
+        G.assert_bits_equal(pa, pb, f"{case} param")
+        for key, val in fast.state[pa].items():
+            if torch.is_tensor(val) and key != "group":
+                G.assert_bits_equal(val, public.state[pb][key], f"{case} {key}") if val.is_cuda else None
+        if "step" in fast.state[pa]:
+            assert int(fast.state[pa]["step"]) == int(public.state[pb]["step"]) == 8
+    assert list(fast.state[a[0]].keys()) == list(public.state[b[0]].keys())
+
+
+def test_step_hooks_still_fire_under_gradient_release(hip_device):
+    model, params = make(torch.bfloat16, hip_device)
+    opt = optimi_amd.AdamW(params, lr=1e-3, gradient_release=True)
+    optimi_amd.prepare_for_gradient_release(model, opt)
+    calls = []
+    handle = opt.register_step_post_hook(lambda o, args, kwargs: calls.append(kwargs.get("param")))
+    loss_step(model, torch.bfloat16, hip_device, torch.Generator().manual_seed(0))
+    assert len(calls) == len(params) and all(c is not None for c in calls)
+    handle.remove()
+    loss_step(model, torch.bfloat16, hip_device, torch.Generator().manual_seed(1))
+    assert len(calls) == len(params)
+    optimi_amd.remove_gradient_release(model)
