@@ -45,7 +45,7 @@ constexpr int kChunkBytes = 16384;        // bytes per array per chunk: the gran
 constexpr int kSub = kChunkBytes / (kThreads * kUnroll * 16);  // workgroups per chunk
 static_assert(kSub >= 1 && kSub * kThreads * kUnroll * 16 == kChunkBytes, "workgroup tile must divide the chunk");
 static_assert(kThreads % 64 == 0 && kThreads <= 1024, "whole wavefronts");
-constexpr int kReduceThreads = 256;       // lanes of the per-tensor finalize workgroup
+constexpr int kReduceThreads = 1024;      // lanes of the per-tensor finalize workgroup
 constexpr int kMaxArrays = 7;   // Adan: p g m diff sq prev kahan
 constexpr int kAbiVersion = 1000;
 
@@ -510,8 +510,18 @@ stable_finalize_kernel(const TensorEntry* __restrict__ table, const TensorEntry 
   const TensorEntry& e = MULTI ? table[blockIdx.x] : single;
   const int64_t first = (MULTI ? e.first_chunk : 0) * kSub;  // one partial per workgroup of pass 1
   const int64_t count = (e.numel + kChunk - 1) / kChunk * kSub;
-  double v = 0.0;
-  for (int64_t c = threadIdx.x; c < count; c += kReduceThreads) v += partials[first + c];
+  // four independent accumulators keep several loads in flight; the order is fixed, so the sum is
+  // the same on every run
+  double v0 = 0.0, v1 = 0.0, v2 = 0.0, v3 = 0.0;
+  int64_t c = threadIdx.x;
+  for (; c + 3 * kReduceThreads < count; c += 4 * kReduceThreads) {
+    v0 += partials[first + c];
+    v1 += partials[first + c + kReduceThreads];
+    v2 += partials[first + c + 2 * kReduceThreads];
+    v3 += partials[first + c + 3 * kReduceThreads];
+  }
+  for (; c < count; c += kReduceThreads) v0 += partials[first + c];
+  double v = (v0 + v1) + (v2 + v3);
   __shared__ double lds[kReduceThreads / 64];
   double total = block_sum<kReduceThreads>(v, lds);
   if (threadIdx.x == 0) {
