@@ -42,7 +42,11 @@ enum optimi_flags {
   OPTIMI_UPDATE = 2,      /* update_parameters; unset = accumulate-only step (optimi/adam.py:308) */
   OPTIMI_DECOUPLE_WD = 4, /* Adam: decoupled decay p*=factor; unset = L2 (optimi/adam.py:373-377) */
   OPTIMI_ADAM_WD = 8,     /* Adan: Adam-style decay before the step (optimi/adan.py:447-448)      */
-  OPTIMI_DECOUPLE_LR = 16 /* StableAdamW: fully decoupled decay (optimi/stableadamw.py:453-457)   */
+  OPTIMI_DECOUPLE_LR = 16,/* StableAdamW: fully decoupled decay (optimi/stableadamw.py:453-457)   */
+  OPTIMI_DAMPENING = 32,  /* SGD: momentum buffer is an EMA, lerp(m, g, 1-momentum) (optimi/sgd.py:352-353) */
+  OPTIMI_RECTIFY = 64,    /* RAdam/Ranger: rho > 5, take the rectified Adam step (optimi/radam.py:269-277) */
+  OPTIMI_LOOKAHEAD = 128  /* Ranger: this step synchronises with the slow weights, step % k == 0
+                             (optimi/ranger.py:452, 471)                                           */
 };
 
 enum optimi_status {
@@ -120,6 +124,31 @@ int optimi_hip_adan_multi(optimi_group* group, int n_tensors, void* const* param
                           double beta1_comp, double beta2, double beta2_comp, double beta3_hat, double beta3_comp,
                           double eps, double weight_decay, uint32_t flags, optimi_stream_t stream);
 
+/* SGD over a list.  Replaces _triton_sgd (optimi/sgd.py:501-543); results follow _single_param_sgd
+ * (optimi/sgd.py:329-372).  exp_avg may be NULL when momentum == 0.  weight_decay as for Adam.
+ * OPTIMI_DAMPENING selects the dampened momentum update. */
+int optimi_hip_sgd_multi(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                         void* const* exp_avg, void* const* kahan_comp, const int64_t* numel, int dtype, double lr,
+                         double momentum, double weight_decay, uint32_t flags, optimi_stream_t stream);
+
+/* RAdam over a list.  Replaces _triton_radam (optimi/radam.py:567-628); results follow
+ * _single_param_radam (optimi/radam.py:368-417).  With OPTIMI_RECTIFY the step is
+ * -lr*rect*m/(sqrt(v)+eps); without it (the first steps) it is -lr*m and `rect` is ignored. */
+int optimi_hip_radam_multi(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                           void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                           const int64_t* numel, int dtype, double lr, double beta1_comp, double beta2_hat,
+                           double beta2_comp, double weight_decay, double eps, double rect, uint32_t flags,
+                           optimi_stream_t stream);
+
+/* Ranger over a list.  Replaces _triton_ranger (optimi/ranger.py:674-745); results follow
+ * _single_param_ranger (optimi/ranger.py:402-473): the RAdam step, then with OPTIMI_LOOKAHEAD the
+ * Lookahead interpolation la += alpha*(p - la), p = la.  la_param is read only on such steps. */
+int optimi_hip_ranger_multi(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                            void* const* exp_avg, void* const* exp_avg_sq, void* const* la_param,
+                            void* const* kahan_comp, const int64_t* numel, int dtype, double lr, double beta1_comp,
+                            double beta2_hat, double beta2_comp, double weight_decay, double eps, double rect,
+                            double alpha, uint32_t flags, optimi_stream_t stream);
+
 /* ---------------------------------------------------------------------------------
  * Per-tensor steps for gradient release: pointers travel as kernel arguments, no table.
  * ------------------------------------------------------------------------------- */
@@ -147,6 +176,22 @@ int optimi_hip_adan_single(void* param, const void* grad, void* exp_avg, void* e
                            void* prev_grad, void* kahan_comp, int64_t numel, int dtype, double lr, double beta1_comp,
                            double beta2, double beta2_comp, double beta3_hat, double beta3_comp, double eps,
                            double weight_decay, uint32_t flags, optimi_stream_t stream);
+
+/* Replaces _single_param_triton_sgd (optimi/sgd.py:545-584). */
+int optimi_hip_sgd_single(void* param, const void* grad, void* exp_avg, void* kahan_comp, int64_t numel, int dtype,
+                          double lr, double momentum, double weight_decay, uint32_t flags, optimi_stream_t stream);
+
+/* Replaces _single_param_triton_radam (optimi/radam.py:630-686). */
+int optimi_hip_radam_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* kahan_comp,
+                            int64_t numel, int dtype, double lr, double beta1_comp, double beta2_hat,
+                            double beta2_comp, double weight_decay, double eps, double rect, uint32_t flags,
+                            optimi_stream_t stream);
+
+/* Replaces _single_param_triton_ranger (optimi/ranger.py:747-810). */
+int optimi_hip_ranger_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* la_param,
+                             void* kahan_comp, int64_t numel, int dtype, double lr, double beta1_comp,
+                             double beta2_hat, double beta2_comp, double weight_decay, double eps, double rect,
+                             double alpha, uint32_t flags, optimi_stream_t stream);
 
 /* ---------------------------------------------------------------------------------
  * Measurement aid (no counterpart in the reference): a plain 16-byte-per-lane copy of

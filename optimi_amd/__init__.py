@@ -7,12 +7,12 @@ served by HIP kernels behind a C ABI (``include/optimi_hip.h``).
 
 __version__ = "0.1.0"
 
-from .functional import adam, adamw, adan, lion, stableadamw
+from .functional import adam, adamw, adan, lion, radam, ranger, sgd, stableadamw
 from .gradient_release import prepare_for_gradient_release, remove_gradient_release
-from .optimizers import Adam, AdamW, Adan, Lion, OptimiOptimizer, StableAdamW
+from .optimizers import SGD, Adam, AdamW, Adan, Lion, OptimiOptimizer, RAdam, Ranger, StableAdamW
 
 __all__ = [
-    "Adam", "AdamW", "Adan", "Lion", "StableAdamW", "OptimiOptimizer",
-    "adam", "adamw", "adan", "lion", "stableadamw",
+    "Adam", "AdamW", "Adan", "Lion", "StableAdamW", "SGD", "RAdam", "Ranger", "OptimiOptimizer",
+    "adam", "adamw", "adan", "lion", "stableadamw", "sgd", "radam", "ranger",
     "prepare_for_gradient_release", "remove_gradient_release",
 ]

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "liboptimi_hip.so")
 
 F32, BF16 = 0, 1
-KAHAN, UPDATE, DECOUPLE_WD, ADAM_WD, DECOUPLE_LR = 1, 2, 4, 8, 16
+KAHAN, UPDATE, DECOUPLE_WD, ADAM_WD, DECOUPLE_LR, DAMPENING, RECTIFY, LOOKAHEAD = 1, 2, 4, 8, 16, 32, 64, 128
 
 _p, _pp, _i, _i64, _u32, _d = C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_int64, C.c_uint32, C.c_double
 _i64p = C.POINTER(C.c_int64)
@@ -29,10 +29,16 @@ PROTOTYPES = {
     "optimi_hip_lion_multi": (_i, [_p, _i, _pp, _pp, _pp, _pp, _i64p, _i, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_stableadamw_multi": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _i64p, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_adan_multi": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _pp, _pp, _i64p, _i, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_sgd_multi": (_i, [_p, _i, _pp, _pp, _pp, _pp, _i64p, _i, _d, _d, _d, _u32, _p]),
+    "optimi_hip_radam_multi": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _i64p, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_ranger_multi": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _pp, _i64p, _i, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_adam_single": (_i, [_p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_lion_single": (_i, [_p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_stableadamw_single": (_i, [_p, _p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_adan_single": (_i, [_p, _p, _p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_sgd_single": (_i, [_p, _p, _p, _p, _i64, _i, _d, _d, _d, _u32, _p]),
+    "optimi_hip_radam_single": (_i, [_p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_ranger_single": (_i, [_p, _p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_copy_probe": (_i, [_p, _p, _i64, _p]),
 }
 

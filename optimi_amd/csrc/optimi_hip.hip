@@ -161,13 +161,14 @@ constexpr uint32_t bit(int i) { return 1u << i; }
 // ------------------------------------------------------------------------------------
 struct AdamScalars {
   Lerp l1;
-  float wd, wd_alpha, b2h, b2c, eps_d, neg_lr;
+  float wd, wd_alpha, b2h, b2c, eps_d, neg_lr, neg_lr_d;
 };
 
 // slots: 0 param, 1 grad, 2 exp_avg, 3 exp_avg_sq, 4 kahan_comp     optimi/adam.py:354-396
 // WD: 0 none, 1 decoupled (p *= wd), 2 L2 (g += wd_alpha * p)
-template <class DT_, bool KAHAN, bool UPDATE, int WD>
-struct AdamOp {
+// TAIL: 0 the Adam step -lr*m/(sqrt(v)+eps); 1 RAdam's unrectified step -lr*m (optimi/radam.py:398-417)
+template <class DT_, bool KAHAN, bool UPDATE, int WD, int TAIL>
+struct AdamTailOp {
   using DT = DT_;
   using Scalars = AdamScalars;
   static constexpr int kArrays = 5;
@@ -185,15 +186,104 @@ struct AdamOp {
     x[2] = m;
     x[3] = v;
     if (UPDATE) {
-      f32x2 d = DT::R2(sqrt2(v));
-      d = DT::R2(d + s.eps_d);
-      if (KAHAN) {
-        f32x2 k = x[4];
+      f32x2 k = KAHAN ? x[4] : p;  // the accumulator the step lands in
+      if (TAIL == 0) {
+        f32x2 d = DT::R2(sqrt2(v));
+        d = DT::R2(d + s.eps_d);
         k = DT::R2(k + div2(m * s.neg_lr, d));
+      } else {
+        k = DT::R2(fma2(m, splat(s.neg_lr_d), k));
+      }
+      if (KAHAN) {
         kahan_commit<DT>(p, k);
         x[4] = k;
       } else {
-        p = DT::R2(p + div2(m * s.neg_lr, d));
+        p = k;
+      }
+      x[0] = p;
+    }
+  }
+};
+template <class DT, bool KAHAN, bool UPDATE, int WD> using AdamOp = AdamTailOp<DT, KAHAN, UPDATE, WD, 0>;
+template <class DT, bool KAHAN, bool UPDATE, int WD> using RAdamEarlyOp = AdamTailOp<DT, KAHAN, UPDATE, WD, 1>;
+
+struct RangerScalars {
+  AdamScalars a;
+  float alpha_d;
+};
+
+// Ranger = the RAdam step, then every k-th step a Lookahead sync with the slow weights.
+// slots: 0 param, 1 grad, 2 exp_avg, 3 exp_avg_sq, 4 kahan_comp, 5 la_param   optimi/ranger.py:402-473
+// LA: this step synchronises (step % k == 0)
+template <class DT_, bool KAHAN, bool UPDATE, int WD, int TAIL, bool LA>
+struct RangerOp {
+  using DT = DT_;
+  using Scalars = RangerScalars;
+  using Inner = AdamTailOp<DT_, KAHAN, UPDATE, WD, TAIL>;
+  static constexpr int kArrays = 6;
+  static constexpr uint32_t kLoad = Inner::kLoad | ((UPDATE && LA) ? bit(5) : 0);
+  static constexpr uint32_t kStore = Inner::kStore | ((UPDATE && LA) ? bit(5) : 0);
+  static constexpr bool kReduce = false;
+  __device__ static __forceinline__ void prepare(Scalars&, int) {}
+  __device__ static __forceinline__ void elem(f32x2* x, const Scalars& s, f32x2& q) {
+    Inner::elem(x, s.a, q);
+    if (UPDATE && LA) {
+      f32x2 p = x[0], la = x[5];
+      f32x2 t = DT::R2(p - la);
+      if (KAHAN) {
+        f32x2 k = x[4];
+        k = DT::R2(fma2(t, splat(s.alpha_d), k));
+        f32x2 old = la;
+        la = DT::R2(old + k);
+        f32x2 err = DT::R2(old - la);
+        k = DT::R2(fma2(err, splat(s.alpha_d), k));
+        x[4] = k;
+      } else {
+        la = DT::R2(fma2(t, splat(s.alpha_d), la));
+      }
+      x[0] = la;
+      x[5] = la;
+    }
+  }
+};
+
+struct SgdScalars {
+  Lerp damp;
+  float wd, wd_alpha, momentum, neg_lr_d;
+};
+
+// slots: 0 param, 1 grad, 2 exp_avg (momentum buffer), 3 kahan_comp          optimi/sgd.py:329-372
+// WD as Adam.  MOM: 0 no momentum (the step uses the gradient), 1 m = m*momentum + g, 2 dampening (lerp)
+template <class DT_, bool KAHAN, bool UPDATE, int WD, int MOM>
+struct SgdOp {
+  using DT = DT_;
+  using Scalars = SgdScalars;
+  static constexpr int kArrays = 4;
+  static constexpr uint32_t kLoad = bit(1) | (MOM ? bit(2) : 0) | (UPDATE ? (bit(0) | (KAHAN ? bit(3) : 0)) : 0);
+  static constexpr uint32_t kStore = (MOM ? bit(2) : 0) | (UPDATE ? (bit(0) | (KAHAN ? bit(3) : 0)) : 0);
+  static constexpr bool kReduce = false;
+  __device__ static __forceinline__ void prepare(Scalars&, int) {}
+  __device__ static __forceinline__ void elem(f32x2* x, const Scalars& s, f32x2&) {
+    f32x2 p = x[0], g = x[1], m = x[2];
+    if (UPDATE && WD == 1) p = DT::R2(p * s.wd);
+    if (UPDATE && WD == 2) g = DT::R2(fma2(p, splat(s.wd_alpha), g));
+    if (MOM == 1) {
+      m = DT::R2(m * s.momentum);
+      m = DT::R2(m + g);
+    } else if (MOM == 2) {
+      m = DT::R2(lerp2(m, g, s.damp));
+    } else {
+      m = g;
+    }
+    if (MOM) x[2] = m;
+    if (UPDATE) {
+      if (KAHAN) {
+        f32x2 k = x[3];
+        k = DT::R2(fma2(m, splat(s.neg_lr_d), k));
+        kahan_commit<DT>(p, k);
+        x[3] = k;
+      } else {
+        p = DT::R2(fma2(m, splat(s.neg_lr_d), p));
       }
       x[0] = p;
     }
@@ -816,6 +906,28 @@ void dispatch(int dtype, bool kahan, bool update, int wd, Fn&& fn) {
   }
 }
 
+// Same selection, handing the choices over as tag types so the caller can add further
+// compile-time parameters of its own: fn(DT{}, bool_c<kahan>, bool_c<update>, int_c<wd>).
+template <bool B> using bool_c = std::integral_constant<bool, B>;
+template <int I> using int_c = std::integral_constant<int, I>;
+
+template <class Fn>
+void dispatch_tags(int dtype, bool kahan, bool update, int wd, Fn&& fn) {
+  auto pick_wd = [&](auto dt, auto kh) {
+    if (wd == 1) fn(dt, kh, bool_c<true>{}, int_c<1>{});
+    else if (wd == 2) fn(dt, kh, bool_c<true>{}, int_c<2>{});
+    else fn(dt, kh, bool_c<true>{}, int_c<0>{});
+  };
+  if (dtype == OPTIMI_BF16) {
+    if (!update) fn(BF16{}, bool_c<false>{}, bool_c<false>{}, int_c<0>{});
+    else if (kahan) pick_wd(BF16{}, bool_c<true>{});
+    else pick_wd(BF16{}, bool_c<false>{});
+  } else {
+    if (!update) fn(F32{}, bool_c<false>{}, bool_c<false>{}, int_c<0>{});
+    else pick_wd(F32{}, bool_c<false>{});
+  }
+}
+
 int single_entry(TensorEntry& e, const void* const* ptrs, int n_arrays, uint32_t need, int64_t numel, int dtype) {
   if (numel < 0) return OPTIMI_ERR_SIZE;
   if (dtype != OPTIMI_F32 && dtype != OPTIMI_BF16) return OPTIMI_ERR_DTYPE;
@@ -846,6 +958,7 @@ AdamScalars adam_scalars(int dtype, double lr, double beta1_comp, double beta2_h
   s.b2c = S(beta2_comp);
   s.eps_d = Sd(eps, dtype);
   s.neg_lr = S(-lr);
+  s.neg_lr_d = Sd(-lr, dtype);
   return s;
 }
 int adam_wd_mode(double weight_decay, uint32_t flags) {
@@ -887,6 +1000,49 @@ int adan_wd_mode(double weight_decay, uint32_t flags) {
 }
 uint32_t adan_need(bool kahan, bool update) {
   return bit(1) | bit(2) | bit(3) | bit(4) | bit(5) | (update ? (bit(0) | (kahan ? bit(6) : 0)) : 0);
+}
+
+SgdScalars sgd_scalars(int dtype, double lr, double momentum, double weight_decay) {
+  SgdScalars s;
+  s.damp = make_lerp(1 - momentum);
+  s.wd = S(weight_decay);
+  s.wd_alpha = Sd(weight_decay, dtype);
+  s.momentum = S(momentum);
+  s.neg_lr_d = Sd(-lr, dtype);
+  return s;
+}
+inline int sgd_mom_mode(double momentum, uint32_t flags) { return momentum != 0 ? ((flags & OPTIMI_DAMPENING) ? 2 : 1) : 0; }
+uint32_t sgd_need(bool kahan, bool update, int mom) {
+  return bit(1) | (mom ? bit(2) : 0) | (update ? (bit(0) | (kahan ? bit(3) : 0)) : 0);
+}
+uint32_t ranger_need(bool kahan, bool update, bool la) { return adam_need(kahan, update) | ((update && la) ? bit(5) : 0); }
+
+// Launches the SGD variant chosen by dtype x kahan x update x decay mode x momentum mode.
+template <class Launch>
+void sgd_dispatch(int dtype, bool kahan, bool update, int wd, int mom, Launch&& launch) {
+  dispatch_tags(dtype, kahan, update, wd, [&](auto dt, auto kh, auto up, auto w) {
+    using DT = decltype(dt);
+    constexpr bool K = decltype(kh)::value, U = decltype(up)::value;
+    constexpr int W = decltype(w)::value;
+    if (mom == 1) launch(SgdOp<DT, K, U, W, 1>{});
+    else if (mom == 2) launch(SgdOp<DT, K, U, W, 2>{});
+    else launch(SgdOp<DT, K, U, W, 0>{});
+  });
+}
+
+// Launches the Ranger variant: ... x rectified or not x Lookahead step or not.
+template <class Launch>
+void ranger_dispatch(int dtype, bool kahan, bool update, int wd, bool rectify, bool la, Launch&& launch) {
+  dispatch_tags(dtype, kahan, update, wd, [&](auto dt, auto kh, auto up, auto w) {
+    using DT = decltype(dt);
+    constexpr bool K = decltype(kh)::value, U = decltype(up)::value;
+    constexpr int W = decltype(w)::value;
+    if (!U) launch(RangerOp<DT, K, U, W, 0, false>{});
+    else if (rectify && la) launch(RangerOp<DT, K, U, W, 0, true>{});
+    else if (rectify) launch(RangerOp<DT, K, U, W, 0, false>{});
+    else if (la) launch(RangerOp<DT, K, U, W, 1, true>{});
+    else launch(RangerOp<DT, K, U, W, 1, false>{});
+  });
 }
 
 StableP1Scalars stable_p1_scalars(int dtype, double beta1_comp, double beta2_hat, double beta2_comp, double eps) {
@@ -1158,6 +1314,121 @@ int optimi_hip_adan_single(void* param, const void* grad, void* exp_avg, void* e
   if (numel == 0) return 0;
   AdanScalars s = adan_scalars(dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay);
   dispatch<AdanOp, 3>(dtype, kahan, update, adan_wd_mode(weight_decay, flags), [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int optimi_hip_sgd_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                         void* const* exp_avg, void* const* kahan_comp, const int64_t* numel, int dtype, double lr,
+                         double momentum, double weight_decay, uint32_t flags, optimi_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const int mom = sgd_mom_mode(momentum, flags);
+  if (!update && !mom) return g ? 0 : OPTIMI_ERR_NULL;  // nothing to accumulate into
+  const void* const* lists[4] = {(const void* const*)param, grad, (const void* const*)exp_avg, (const void* const*)kahan_comp};
+  int rc = prepare_tables(g, n_tensors, lists, 4, sgd_need(kahan, update, mom), numel, dtype, stream);
+  if (rc) return rc;
+  if (g->n_chunks == 0) return 0;
+  SgdScalars s = sgd_scalars(dtype, lr, momentum, weight_decay);
+  sgd_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), mom, [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
+  return note_launch(g, stream);
+}
+
+int optimi_hip_sgd_single(void* param, const void* grad, void* exp_avg, void* kahan_comp, int64_t numel, int dtype,
+                          double lr, double momentum, double weight_decay, uint32_t flags, optimi_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const int mom = sgd_mom_mode(momentum, flags);
+  const void* ptrs[4] = {param, grad, exp_avg, kahan_comp};
+  TensorEntry e;
+  int rc = single_entry(e, ptrs, 4, sgd_need(kahan, update, mom), numel, dtype);
+  if (rc) return rc;
+  if (numel == 0 || (!update && !mom)) return 0;
+  SgdScalars s = sgd_scalars(dtype, lr, momentum, weight_decay);
+  sgd_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), mom, [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int optimi_hip_radam_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                           void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                           const int64_t* numel, int dtype, double lr, double beta1_comp, double beta2_hat,
+                           double beta2_comp, double weight_decay, double eps, double rect, uint32_t flags,
+                           optimi_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const bool rectify = (flags & OPTIMI_RECTIFY) != 0;
+  const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
+                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
+  int rc = prepare_tables(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, stream);
+  if (rc) return rc;
+  if (g->n_chunks == 0) return 0;
+  AdamScalars s = adam_scalars(dtype, rectify ? lr * rect : lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  const int wd = adam_wd_mode(weight_decay, flags);
+  if (rectify || !update) dispatch<AdamOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
+  else dispatch<RAdamEarlyOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
+  return note_launch(g, stream);
+}
+
+int optimi_hip_radam_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* kahan_comp,
+                            int64_t numel, int dtype, double lr, double beta1_comp, double beta2_hat,
+                            double beta2_comp, double weight_decay, double eps, double rect, uint32_t flags,
+                            optimi_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const bool rectify = (flags & OPTIMI_RECTIFY) != 0;
+  const void* ptrs[5] = {param, grad, exp_avg, exp_avg_sq, kahan_comp};
+  TensorEntry e;
+  int rc = single_entry(e, ptrs, 5, adam_need(kahan, update), numel, dtype);
+  if (rc) return rc;
+  if (numel == 0) return 0;
+  AdamScalars s = adam_scalars(dtype, rectify ? lr * rect : lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  const int wd = adam_wd_mode(weight_decay, flags);
+  if (rectify || !update) dispatch<AdamOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
+  else dispatch<RAdamEarlyOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+int optimi_hip_ranger_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                            void* const* exp_avg, void* const* exp_avg_sq, void* const* la_param,
+                            void* const* kahan_comp, const int64_t* numel, int dtype, double lr, double beta1_comp,
+                            double beta2_hat, double beta2_comp, double weight_decay, double eps, double rect,
+                            double alpha, uint32_t flags, optimi_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const bool rectify = (flags & OPTIMI_RECTIFY) != 0, la = (flags & OPTIMI_LOOKAHEAD) != 0;
+  const void* const* lists[6] = {(const void* const*)param, grad, (const void* const*)exp_avg,
+                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp,
+                                 (const void* const*)la_param};
+  int rc = prepare_tables(g, n_tensors, lists, 6, ranger_need(kahan, update, la), numel, dtype, stream);
+  if (rc) return rc;
+  if (g->n_chunks == 0) return 0;
+  RangerScalars s;
+  s.a = adam_scalars(dtype, rectify ? lr * rect : lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  s.alpha_d = Sd(alpha, dtype);
+  ranger_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), rectify, la,
+                  [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
+  return note_launch(g, stream);
+}
+
+int optimi_hip_ranger_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* la_param,
+                             void* kahan_comp, int64_t numel, int dtype, double lr, double beta1_comp,
+                             double beta2_hat, double beta2_comp, double weight_decay, double eps, double rect,
+                             double alpha, uint32_t flags, optimi_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const bool rectify = (flags & OPTIMI_RECTIFY) != 0, la = (flags & OPTIMI_LOOKAHEAD) != 0;
+  const void* ptrs[6] = {param, grad, exp_avg, exp_avg_sq, kahan_comp, la_param};
+  TensorEntry e;
+  int rc = single_entry(e, ptrs, 6, ranger_need(kahan, update, la), numel, dtype);
+  if (rc) return rc;
+  if (numel == 0) return 0;
+  RangerScalars s;
+  s.a = adam_scalars(dtype, rectify ? lr * rect : lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  s.alpha_d = Sd(alpha, dtype);
+  ranger_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), rectify, la,
+                  [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
   HIP_TRY(hipGetLastError());
   return 0;
 }

@@ -181,6 +181,67 @@ void adan_multi(Group& group, const TensorList& params, const TensorList& grads,
                "optimi_hip_adan_multi");
 }
 
+// Momentum buffers: absent (None or a one-element placeholder) when SGD runs without momentum.
+PtrList gather_optional(const TensorList& params, const OptTensorList& list, bool needed, const char* name) {
+  PtrList out;
+  if (!needed) return out;
+  TORCH_CHECK(list.size() == params.size(), "optimi_amd: ", name, " has ", list.size(), " tensors, params has ", params.size());
+  out.v.reserve(list.size());
+  for (size_t i = 0; i < list.size(); ++i) {
+    TORCH_CHECK(list[i].has_value(), "optimi_amd: ", name, " is needed but missing");
+    check_like(params[i], *list[i], name);
+    out.v.push_back(list[i]->data_ptr());
+  }
+  return out;
+}
+
+void sgd_multi(Group& group, const TensorList& params, const TensorList& grads, const OptTensorList& exp_avgs,
+               const OptTensorList& kahan_comps, double lr, double momentum, double weight_decay, uint32_t flags) {
+  if (params.empty()) return;
+  Prepared pr = prepare(params, flags);
+  PtrList g = gather(params, grads, "grad");
+  PtrList m = gather_optional(params, exp_avgs, momentum != 0, "exp_avg");
+  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
+  check_status(optimi_hip_sgd_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(),
+                                    momentum != 0 ? m.data() : nullptr, pr.kahan ? k.data() : nullptr, pr.numel.data(),
+                                    pr.dtype, lr, momentum, weight_decay, flags,
+                                    c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+               "optimi_hip_sgd_multi");
+}
+
+void radam_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
+                 const TensorList& exp_avg_sqs, const OptTensorList& kahan_comps, double lr, double beta1_comp,
+                 double beta2_hat, double beta2_comp, double weight_decay, double eps, double rect, uint32_t flags) {
+  if (params.empty()) return;
+  Prepared pr = prepare(params, flags);
+  PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
+  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
+  check_status(optimi_hip_radam_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
+                                      pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp, beta2_hat,
+                                      beta2_comp, weight_decay, eps, rect, flags,
+                                      c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+               "optimi_hip_radam_multi");
+}
+
+void ranger_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
+                  const TensorList& exp_avg_sqs, const TensorList& la_params, const OptTensorList& kahan_comps, double lr,
+                  double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay, double eps, double rect,
+                  double alpha, uint32_t flags) {
+  if (params.empty()) return;
+  Prepared pr = prepare(params, flags);
+  PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
+  PtrList la = gather(params, la_params, "la_param");
+  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
+  check_status(optimi_hip_ranger_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
+                                       la.data(), pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp,
+                                       beta2_hat, beta2_comp, weight_decay, eps, rect, alpha, flags,
+                                       c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+               "optimi_hip_ranger_multi");
+}
+
 // ---- per-tensor entry points (gradient release) --------------------------------------
 struct One {
   int dtype;
@@ -339,6 +400,96 @@ void adan_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m,
               flags);
 }
 
+void sgd_single(const at::Tensor& p, const at::Tensor& g, const std::optional<at::Tensor>& m,
+                const std::optional<at::Tensor>& kahan_comp, double lr, double momentum, double weight_decay, uint32_t flags) {
+  One o = prepare_one(p, kahan_comp, flags);
+  check_like(p, g, "grad");
+  void* mp = nullptr;
+  if (momentum != 0) {
+    TORCH_CHECK(m.has_value(), "optimi_amd: momentum is on but the momentum buffer is missing");
+    check_like(p, *m, "exp_avg");
+    mp = m->data_ptr();
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(p.device());
+  check_status(optimi_hip_sgd_single(p.data_ptr(), g.data_ptr(), mp, o.k, p.numel(), o.dtype, lr, momentum, weight_decay,
+                                     flags, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+               "optimi_hip_sgd_single");
+}
+
+void radam_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
+                  const std::optional<at::Tensor>& kahan_comp, double lr, double beta1_comp, double beta2_hat,
+                  double beta2_comp, double weight_decay, double eps, double rect, uint32_t flags) {
+  One o = prepare_one(p, kahan_comp, flags);
+  check_like(p, g, "grad");
+  check_like(p, m, "exp_avg");
+  check_like(p, v, "exp_avg_sq");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(p.device());
+  check_status(optimi_hip_radam_single(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), o.k, p.numel(), o.dtype, lr,
+                                       beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, rect, flags,
+                                       c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+               "optimi_hip_radam_single");
+}
+
+void ranger_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v, const at::Tensor& la,
+                   const std::optional<at::Tensor>& kahan_comp, double lr, double beta1_comp, double beta2_hat,
+                   double beta2_comp, double weight_decay, double eps, double rect, double alpha, uint32_t flags) {
+  One o = prepare_one(p, kahan_comp, flags);
+  check_like(p, g, "grad");
+  check_like(p, m, "exp_avg");
+  check_like(p, v, "exp_avg_sq");
+  check_like(p, la, "la_param");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(p.device());
+  check_status(optimi_hip_ranger_single(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), la.data_ptr(), o.k, p.numel(),
+                                        o.dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, rect, alpha, flags,
+                                        c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+               "optimi_hip_ranger_single");
+}
+
+// RAdam's variance rectification term; negative = not yet rectified (optimi/radam.py:269-277).
+double rectification(double beta2, int64_t step) {
+  const double rho_inf = 2 / (1 - beta2) - 1;
+  const double bt = std::pow(beta2, (double)step);
+  const double rho = rho_inf - 2 * (double)step * bt / (1 - bt);
+  if (rho > 5) return std::sqrt(((rho - 4) * (rho - 2) * rho_inf) / ((rho_inf - 4) * (rho_inf - 2) * rho));
+  return -1.0;
+}
+
+void sgd_release(const at::Tensor& p, const at::Tensor& g, const std::optional<at::Tensor>& m,
+                 const std::optional<at::Tensor>& k, double lr, double momentum, double weight_decay, bool dampening,
+                 bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update) {
+  if (weight_decay != 0) {
+    if (decouple_lr) weight_decay = 1 - (lr / max_lr.value()) * weight_decay;
+    else if (decouple_wd) weight_decay = 1 - lr * weight_decay;
+  }
+  const uint32_t flags = base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u) |
+                         (dampening ? OPTIMI_DAMPENING : 0u);
+  sgd_single(p, grad_like(p, g), momentum != 0 ? real_kahan(p, m) : std::nullopt, real_kahan(p, k), lr, momentum, weight_decay, flags);
+}
+
+void ranger_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
+                    const std::optional<at::Tensor>& la, const std::optional<at::Tensor>& k, const at::Tensor& step, double lr,
+                    double beta1, double beta2, double weight_decay, double eps, int64_t sync_every, double alpha,
+                    bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update) {
+  // la = None makes this RAdam (optimi/radam.py:214-322); with la it is Ranger (optimi/ranger.py:230-344)
+  const int64_t t = tick(step);
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
+  const double rect = rectification(beta2, t);
+  if (weight_decay != 0) {
+    if (decouple_lr) weight_decay = 1 - (lr / max_lr.value()) * weight_decay;
+    else if (decouple_wd) weight_decay = 1 - lr * weight_decay;
+  }
+  uint32_t flags = base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u) |
+                   (rect >= 0 ? OPTIMI_RECTIFY : 0u);
+  if (la.has_value()) {
+    if (t % sync_every == 0) flags |= OPTIMI_LOOKAHEAD;
+    ranger_single(p, grad_like(p, g), m, v, *la, real_kahan(p, k), lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps,
+                  rect >= 0 ? rect : 0.0, alpha, flags);
+  } else {
+    radam_single(p, grad_like(p, g), m, v, real_kahan(p, k), lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps,
+                 rect >= 0 ? rect : 0.0, flags);
+  }
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
@@ -348,6 +499,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.attr("DECOUPLE_WD") = (uint32_t)OPTIMI_DECOUPLE_WD;
   mod.attr("ADAM_WD") = (uint32_t)OPTIMI_ADAM_WD;
   mod.attr("DECOUPLE_LR") = (uint32_t)OPTIMI_DECOUPLE_LR;
+  mod.attr("DAMPENING") = (uint32_t)OPTIMI_DAMPENING;
+  mod.attr("RECTIFY") = (uint32_t)OPTIMI_RECTIFY;
+  mod.attr("LOOKAHEAD") = (uint32_t)OPTIMI_LOOKAHEAD;
   mod.def("abi_version", &optimi_hip_version);
   py::class_<Group>(mod, "Group").def(py::init<>());
   mod.def("adam_multi", &adam_multi);
@@ -363,4 +517,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.def("stableadamw_release", &stableadamw_release);
   mod.def("adan_release", &adan_release);
   mod.def("debias_beta", &debias_beta);
+  mod.def("rectification", &rectification);
+  mod.def("sgd_multi", &sgd_multi);
+  mod.def("radam_multi", &radam_multi);
+  mod.def("ranger_multi", &ranger_multi);
+  mod.def("sgd_single", &sgd_single);
+  mod.def("radam_single", &radam_single);
+  mod.def("ranger_single", &ranger_single);
+  mod.def("sgd_release", &sgd_release);
+  mod.def("ranger_release", &ranger_release);
 }

@@ -1,7 +1,9 @@
-"""Functional optimizer steps: ``adam``, ``adamw``, ``lion``, ``stableadamw``, ``adan``.
+"""Functional optimizer steps: ``adam``, ``adamw``, ``lion``, ``stableadamw``, ``adan``, ``sgd``,
+``radam``, ``ranger``.
 
 Same keyword signatures as the reference's functional forms (optimi/adam.py:213-234,
-adamw.py:78-98, lion.py:187-204, stableadamw.py:277-299, adan.py:236-260).  Each forms the
+adamw.py:78-98, lion.py:187-204, stableadamw.py:277-299, adan.py:236-260, sgd.py:213-231,
+radam.py:214-235, ranger.py:230-254).  Each forms the
 step scalars in Python doubles exactly where the reference does, then hands the tensors
 to the HIP backend: one launch for a list, the per-tensor entry point when
 ``gradient_release=True``.  ``triton=True`` selects that backend; it is the only one in
@@ -11,15 +13,16 @@ path behind the caller's back.
 
 from __future__ import annotations
 
+import math
 from collections import defaultdict
 
 import torch
 from torch import Tensor
 
 from . import backend
-from .utils import debias_beta
+from .utils import debias, debias_beta
 
-__all__ = ["adam", "adamw", "lion", "stableadamw", "adan"]
+__all__ = ["adam", "adamw", "lion", "stableadamw", "adan", "sgd", "radam", "ranger"]
 
 _LOW_PRECISION = (torch.float16, torch.bfloat16)
 
@@ -341,6 +344,193 @@ def adan(
         ext.adan_multi(grp, _pick(params, idxs), _pick(grads, idxs), _pick(exp_avgs, idxs), _pick(exp_avg_diffs, idxs),
                        _pick(exp_avg_sqs, idxs), _pick(prev_grads, idxs),
                        [_real_kahan(params[i], kahan_comps[i]) for i in idxs], *scalars)
+
+
+# --------------------------------------------------------------------------------------
+# SGD
+# --------------------------------------------------------------------------------------
+def sgd(
+    params: list[Tensor] | Tensor,
+    grads: list[Tensor] | Tensor,
+    exp_avgs: list[Tensor | None] | Tensor | None,
+    kahan_comps: list[Tensor | None] | Tensor | None = None,
+    *,
+    lr: float,
+    momentum: float,
+    weight_decay: float,
+    dampening: bool,
+    decouple_wd: bool,
+    decouple_lr: bool = False,
+    max_lr: float | None = None,
+    kahan_sum: bool = False,
+    foreach: bool = False,
+    triton: bool = False,
+    gradient_release: bool = False,
+    optimizer_accumulation: bool = False,
+    _groups=None,
+):
+    """Functional API to apply a SGD or SGDW optimization step (optimi/sgd.py:213-298)."""
+    _require_hip_backend(triton, foreach, gradient_release)
+    ext = backend.ext()
+
+    if weight_decay != 0:
+        if decouple_lr:
+            weight_decay = 1 - (lr / max_lr) * weight_decay
+        elif decouple_wd:
+            weight_decay = 1 - lr * weight_decay
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation,
+                   DECOUPLE_WD=decouple_wd or decouple_lr, DAMPENING=dampening)
+    scalars = (lr, momentum, weight_decay, flags)
+
+    single = isinstance(params, Tensor)
+    if kahan_comps is None:
+        kahan_comps = [None] * (1 if single else len(params))
+    if exp_avgs is None:
+        exp_avgs = [None] * (1 if single else len(params))
+    params, grads, exp_avgs, kahan_comps = _as_lists(params, grads, exp_avgs, kahan_comps)
+    grads = _grads_like(params, grads)
+    # without momentum the buffer is None or a one-element placeholder (optimi/sgd.py:103-106)
+    moms = [_real_kahan(p, m) if momentum != 0 else None for p, m in zip(params, exp_avgs)]
+
+    if gradient_release:
+        for p, g, m, k in zip(params, grads, moms, kahan_comps):
+            backend.check_supported(p)
+            ext.sgd_single(p, g, m, _real_kahan(p, k), *scalars)
+        return
+    for (device, dtype), idxs in _buckets(params).items():
+        grp = _workspace(_groups, device, dtype, "sgd")
+        ext.sgd_multi(grp, _pick(params, idxs), _pick(grads, idxs), _pick(moms, idxs),
+                      [_real_kahan(params[i], kahan_comps[i]) for i in idxs], *scalars)
+
+
+# --------------------------------------------------------------------------------------
+# RAdam and Ranger
+# --------------------------------------------------------------------------------------
+def _rectification(beta2: float, step: int) -> float | None:
+    """Variance rectification term once the approximated SMA is longer than 5, else None
+    (optimi/radam.py:269-277)."""
+    rho_inf = 2 / (1 - beta2) - 1
+    rho = rho_inf - 2 * step * (beta2**step) / debias(beta2, step)
+    if rho > 5:
+        return math.sqrt(((rho - 4) * (rho - 2) * rho_inf) / ((rho_inf - 4) * (rho_inf - 2) * rho))
+    return None
+
+
+def radam(
+    params: list[Tensor],
+    grads: list[Tensor],
+    exp_avgs: list[Tensor],
+    exp_avg_sqs: list[Tensor],
+    kahan_comps: list[Tensor | None] | None = None,
+    *,
+    lr: float,
+    beta1: float,
+    beta2: float,
+    weight_decay: float,
+    eps: float,
+    step: Tensor,
+    decouple_wd: bool,
+    decouple_lr: bool = False,
+    max_lr: float | None = None,
+    kahan_sum: bool = False,
+    foreach: bool = False,
+    triton: bool = False,
+    gradient_release: bool = False,
+    optimizer_accumulation: bool = False,
+    _groups=None,
+):
+    """Functional API to apply an RAdam optimization step (optimi/radam.py:214-322)."""
+    _require_hip_backend(triton, foreach, gradient_release)
+    ext = backend.ext()
+
+    t = _tick(step)
+    beta1_hat = debias_beta(beta1, t)
+    beta2_hat = debias_beta(beta2, t)
+    rect = _rectification(beta2, t)
+    if weight_decay != 0:
+        if decouple_lr:
+            weight_decay = 1 - (lr / max_lr) * weight_decay
+        elif decouple_wd:
+            weight_decay = 1 - lr * weight_decay
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation,
+                   DECOUPLE_WD=decouple_wd or decouple_lr, RECTIFY=rect is not None)
+    scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps, rect if rect is not None else 0.0, flags)
+
+    if kahan_comps is None:
+        kahan_comps = [None] * (1 if isinstance(params, Tensor) else len(params))
+    params, grads, exp_avgs, exp_avg_sqs, kahan_comps = _as_lists(params, grads, exp_avgs, exp_avg_sqs, kahan_comps)
+    grads = _grads_like(params, grads)
+
+    if gradient_release:
+        for p, g, m, v, k in zip(params, grads, exp_avgs, exp_avg_sqs, kahan_comps):
+            backend.check_supported(p)
+            ext.radam_single(p, g, m, v, _real_kahan(p, k), *scalars)
+        return
+    for (device, dtype), idxs in _buckets(params).items():
+        grp = _workspace(_groups, device, dtype, "radam")
+        ext.radam_multi(grp, _pick(params, idxs), _pick(grads, idxs), _pick(exp_avgs, idxs), _pick(exp_avg_sqs, idxs),
+                        [_real_kahan(params[i], kahan_comps[i]) for i in idxs], *scalars)
+
+
+def ranger(
+    params: list[Tensor],
+    grads: list[Tensor],
+    exp_avgs: list[Tensor],
+    exp_avg_sqs: list[Tensor],
+    la_params: list[Tensor],
+    kahan_comps: list[Tensor | None] | None = None,
+    *,
+    lr: float,
+    beta1: float,
+    beta2: float,
+    weight_decay: float,
+    eps: float,
+    k: int,
+    alpha: float,
+    step: Tensor,
+    decouple_wd: bool,
+    decouple_lr: bool = False,
+    max_lr: float | None = None,
+    kahan_sum: bool = False,
+    foreach: bool = False,
+    triton: bool = False,
+    gradient_release: bool = False,
+    optimizer_accumulation: bool = False,
+    _groups=None,
+):
+    """Functional API to apply a Ranger optimization step: RAdam plus Lookahead every ``k`` steps
+    (optimi/ranger.py:230-344)."""
+    _require_hip_backend(triton, foreach, gradient_release)
+    ext = backend.ext()
+
+    t = _tick(step)
+    beta1_hat = debias_beta(beta1, t)
+    beta2_hat = debias_beta(beta2, t)
+    rect = _rectification(beta2, t)
+    if weight_decay != 0:
+        if decouple_lr:
+            weight_decay = 1 - (lr / max_lr) * weight_decay
+        elif decouple_wd:
+            weight_decay = 1 - lr * weight_decay
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation,
+                   DECOUPLE_WD=decouple_wd or decouple_lr, RECTIFY=rect is not None, LOOKAHEAD=t % k == 0)
+    scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps, rect if rect is not None else 0.0, alpha, flags)
+
+    if kahan_comps is None:
+        kahan_comps = [None] * (1 if isinstance(params, Tensor) else len(params))
+    params, grads, exp_avgs, exp_avg_sqs, la_params, kahan_comps = _as_lists(
+        params, grads, exp_avgs, exp_avg_sqs, la_params, kahan_comps)
+    grads = _grads_like(params, grads)
+
+    if gradient_release:
+        for p, g, m, v, la, kc in zip(params, grads, exp_avgs, exp_avg_sqs, la_params, kahan_comps):
+            backend.check_supported(p)
+            ext.ranger_single(p, g, m, v, la, _real_kahan(p, kc), *scalars)
+        return
+    for (device, dtype), idxs in _buckets(params).items():
+        grp = _workspace(_groups, device, dtype, "ranger")
+        ext.ranger_multi(grp, _pick(params, idxs), _pick(grads, idxs), _pick(exp_avgs, idxs), _pick(exp_avg_sqs, idxs),
+                         _pick(la_params, idxs), [_real_kahan(params[i], kahan_comps[i]) for i in idxs], *scalars)
 
 
 # --------------------------------------------------------------------------------------

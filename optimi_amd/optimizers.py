@@ -23,7 +23,7 @@ from torch.optim import optimizer as _torch_optimizer
 from . import backend
 from . import functional as F
 
-__all__ = ["OptimiOptimizer", "Adam", "AdamW", "Lion", "StableAdamW", "Adan"]
+__all__ = ["OptimiOptimizer", "Adam", "AdamW", "Lion", "StableAdamW", "Adan", "SGD", "RAdam", "Ranger"]
 
 _LOW_PRECISION = (torch.float16, torch.bfloat16)
 
@@ -539,3 +539,194 @@ class Adan(OptimiOptimizer):
                          state["kahan_comp"], state["step"], group["lr"], group["beta1"], group["beta2"], group["beta3"],
                          group["weight_decay"], group["eps"], group["decouple_lr"], group["max_lr"], False,
                          bool(group["kahan_sum"]), update)
+
+
+class SGD(OptimiOptimizer):
+    """SGD optimizer. Optionally with momentum and decoupled weight decay.
+
+    Args:
+        params: Iterable of parameters to optimize or dicts defining parameter groups
+        lr: Learning rate
+        momentum: Momentum factor. Gradient moving average coefficient if `dampening` is True
+            (default: 0)
+        weight_decay: Weight decay coefficient. If `decouple_wd` and `decouple_lr` are False,
+            applies L2 penalty (default: 0)
+        dampening: Use dampening for momentum update (default: False)
+        decouple_wd: Apply decoupled weight decay instead of L2 penalty (default: False)
+        decouple_lr: Apply fully decoupled weight decay instead of L2 penalty (default: False)
+        max_lr: Maximum scheduled learning rate. Set if `lr` is not the maximum scheduled learning
+            rate and `decouple_lr` is True (default: None)
+        torch_init: Initialize momentum buffer with first gradient instead of zeroes. Enable to
+            match PyTorch SGD when using dampening (default: False)
+        kahan_sum, foreach, triton, gradient_release: as `Adam`
+    """
+
+    _has_step = False
+
+    def __init__(
+        self,
+        params: Iterable[Tensor] | Iterable[dict],
+        lr: float,
+        momentum: float = 0,
+        weight_decay: float = 0,
+        dampening: bool = False,
+        decouple_wd: bool = False,
+        decouple_lr: bool = False,
+        max_lr: float | None = None,
+        torch_init: bool = False,
+        kahan_sum: bool | None = None,
+        foreach: bool | None = None,
+        triton: bool | None = None,
+        gradient_release: bool = False,
+    ):
+        if not 0.0 <= momentum < 1.0:
+            raise ValueError(f"Invalid momentum: {momentum=}")
+        defaults = dict(lr=lr, momentum=momentum, weight_decay=weight_decay, dampening=dampening,
+                        decouple_wd=decouple_wd, decouple_lr=decouple_lr, max_lr=max_lr, kahan_sum=kahan_sum,
+                        torch_init=torch_init, foreach=foreach, triton=triton, gradient_release=gradient_release,
+                        setup=False)
+        super().__init__(params, defaults)
+
+    def _extra_state(self, group, state, param):
+        # the momentum buffer: first gradient (torch's convention, after L2 decay), zeros, or absent
+        # (optimi/sgd.py:97-107)
+        if group["dampening"] and group["torch_init"]:
+            state["exp_avg"] = param.grad.detach().clone()
+            if group["weight_decay"] != 0 and not group["decouple_lr"] and not group["decouple_wd"]:
+                # exp_avg.add_(param, alpha=wd) as ATen's CPU kernel computes it, which defines the
+                # results: alpha narrowed to the tensor dtype, one fused multiply-add, one rounding
+                # (float64 holds the product and the sum of two narrow floats exactly)
+                alpha = float(torch.tensor(group["weight_decay"], dtype=param.dtype))
+                fused = state["exp_avg"].double().add_(param.double(), alpha=alpha)
+                state["exp_avg"] = fused.float().to(param.dtype)
+        elif group["momentum"] != 0:
+            state["exp_avg"] = torch.zeros_like(param, memory_format=torch.preserve_format)
+        elif group["triton"]:
+            state["exp_avg"] = torch.zeros(1, dtype=param.dtype, device=param.device)
+        else:
+            state["exp_avg"] = None
+
+    def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
+        F.sgd(params, grads, _col(states, "exp_avg"), _col(states, "kahan_comp"), lr=group["lr"],
+              momentum=group["momentum"], weight_decay=group["weight_decay"], dampening=group["dampening"],
+              decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"], max_lr=group["max_lr"],
+              kahan_sum=group["kahan_sum"], foreach=False, triton=True, gradient_release=gradient_release,
+              optimizer_accumulation=accumulate, _groups=self._hip_groups)
+
+    def _release_call(self, ext, group, state, param, grad, update):
+        ext.sgd_release(param, grad, state["exp_avg"], state["kahan_comp"], group["lr"], group["momentum"],
+                        group["weight_decay"], group["dampening"], group["decouple_wd"], group["decouple_lr"],
+                        group["max_lr"], bool(group["kahan_sum"]), update)
+
+
+class RAdam(OptimiOptimizer):
+    """Rectified Adam optimizer. Optionally with decoupled weight decay.
+
+    Args:
+        params: Iterable of parameters to optimize or dicts defining parameter groups
+        lr: Learning rate
+        betas: Coefficients for gradient and squared gradient moving averages (default: (0.9, 0.99))
+        weight_decay: Weight decay coefficient. If `decouple_wd` and `decouple_lr` are False,
+            applies L2 penalty (default: 0)
+        eps: Added to denominator to improve numerical stability (default: 1e-6)
+        decouple_wd: Apply decoupled weight decay instead of L2 penalty (default: False)
+        decouple_lr, max_lr, kahan_sum, foreach, triton, gradient_release: as `Adam`
+    """
+
+    _moment_keys = ("exp_avg", "exp_avg_sq")
+
+    def __init__(
+        self,
+        params: Iterable[Tensor] | Iterable[dict],
+        lr: float,
+        betas: tuple[float, float] = (0.9, 0.99),
+        weight_decay: float = 0,
+        eps: float = 1e-6,
+        decouple_wd: bool = False,
+        decouple_lr: bool = False,
+        max_lr: float | None = None,
+        kahan_sum: bool | None = None,
+        foreach: bool | None = None,
+        triton: bool | None = None,
+        gradient_release: bool = False,
+    ):
+        _check_betas(betas)
+        if not 0.0 <= eps:
+            raise ValueError(f"Invalid epsilon: {eps=}")
+        defaults = dict(lr=lr, beta1=betas[0], beta2=betas[1], eps=eps, weight_decay=weight_decay,
+                        decouple_wd=decouple_wd, decouple_lr=decouple_lr, max_lr=max_lr, kahan_sum=kahan_sum,
+                        foreach=foreach, triton=triton, gradient_release=gradient_release, setup=False)
+        super().__init__(params, defaults)
+
+    def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
+        F.radam(params, grads, _col(states, "exp_avg"), _col(states, "exp_avg_sq"), _col(states, "kahan_comp"),
+                lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"], weight_decay=group["weight_decay"],
+                eps=group["eps"], step=step, decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"],
+                max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
+                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
+
+    def _release_call(self, ext, group, state, param, grad, update):
+        ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], None, state["kahan_comp"], state["step"],
+                           group["lr"], group["beta1"], group["beta2"], group["weight_decay"], group["eps"], 1, 0.0,
+                           group["decouple_wd"], group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update)
+
+
+class Ranger(OptimiOptimizer):
+    """Ranger optimizer. RAdam with Lookahead.
+
+    Args:
+        params: Iterable of parameters to optimize or dicts defining parameter groups
+        lr: Learning rate
+        betas: Coefficients for gradient and squared gradient moving averages (default: (0.9, 0.99))
+        weight_decay: Weight decay coefficient. If `decouple_wd` and `decouple_lr` are False,
+            applies L2 penalty (default: 0)
+        eps: Added to denominator to improve numerical stability (default: 1e-6)
+        k: Lookahead synchronization period (default: 6)
+        alpha: Lookahead weight interpolation coefficient (default: 0.5)
+        decouple_wd: Apply decoupled weight decay instead of L2 penalty (default: True)
+        decouple_lr, max_lr, kahan_sum, foreach, triton, gradient_release: as `Adam`
+    """
+
+    _moment_keys = ("exp_avg", "exp_avg_sq")
+
+    def __init__(
+        self,
+        params: Iterable[Tensor] | Iterable[dict],
+        lr: float,
+        betas: tuple[float, float] = (0.9, 0.99),
+        weight_decay: float = 0,
+        eps: float = 1e-6,
+        k: int = 6,
+        alpha: float = 0.5,
+        decouple_wd: bool = True,
+        decouple_lr: bool = False,
+        max_lr: float | None = None,
+        kahan_sum: bool | None = None,
+        foreach: bool | None = None,
+        triton: bool | None = None,
+        gradient_release: bool = False,
+    ):
+        _check_betas(betas)
+        if not 0.0 <= eps:
+            raise ValueError(f"Invalid epsilon: {eps=}")
+        defaults = dict(lr=lr, beta1=betas[0], beta2=betas[1], eps=eps, weight_decay=weight_decay, k=k, alpha=alpha,
+                        decouple_wd=decouple_wd, decouple_lr=decouple_lr, max_lr=max_lr, kahan_sum=kahan_sum,
+                        foreach=foreach, triton=triton, gradient_release=gradient_release, setup=False)
+        super().__init__(params, defaults)
+
+    def _extra_state(self, group, state, param):
+        state["la_param"] = param.data.clone()  # the slow weights start at the parameters (optimi/ranger.py:142)
+
+    def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
+        F.ranger(params, grads, _col(states, "exp_avg"), _col(states, "exp_avg_sq"), _col(states, "la_param"),
+                 _col(states, "kahan_comp"), lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"],
+                 weight_decay=group["weight_decay"], eps=group["eps"], k=group["k"], alpha=group["alpha"], step=step,
+                 decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"], max_lr=group["max_lr"],
+                 kahan_sum=group["kahan_sum"], foreach=False, triton=True, gradient_release=gradient_release,
+                 optimizer_accumulation=accumulate, _groups=self._hip_groups)
+
+    def _release_call(self, ext, group, state, param, grad, update):
+        ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], state["la_param"], state["kahan_comp"],
+                           state["step"], group["lr"], group["beta1"], group["beta2"], group["weight_decay"],
+                           group["eps"], group["k"], group["alpha"], group["decouple_wd"], group["decouple_lr"],
+                           group["max_lr"], bool(group["kahan_sum"]), update)

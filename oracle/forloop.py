@@ -23,12 +23,20 @@ function                   pinned by
 ``stableadamw_tensor``     golden fixtures; rms<=1 reduces to ``adam_tensor``;
                            scalar C emulator
 ``adan_tensor``            golden fixtures; t=1 closed form; scalar C emulator
+``sgd_tensor``             golden fixtures; torch.optim.SGD equivalence in fp32;
+                           scalar C emulator
+``radam_tensor``           golden fixtures; torch.optim.RAdam equivalence in fp32;
+                           scalar C emulator
+``ranger_tensor``          golden fixtures; float64 Lookahead-over-RAdam
+                           restatement; scalar C emulator
 functional ``adam`` …      golden fixtures (class API and gradient-release /
                            accumulation runs of the reference)
 =========================  ====================================================
 """
 
 from __future__ import annotations
+
+import math
 
 import torch
 from torch import Tensor
@@ -247,6 +255,145 @@ def adan(params, grads, exp_avgs, exp_avg_diffs, exp_avg_sqs, prev_grads, kahan_
 
 
 # ----------------------------------------------------------------------------
+# SGD, one tensor                                 optimi/sgd.py:329-372
+# ----------------------------------------------------------------------------
+def sgd_tensor(param, grad, exp_avg, kahan_comp, *, lr, momentum, weight_decay, dampening, decouple_wd,
+               kahan_sum=False, update_parameters=True):
+    if weight_decay != 0 and update_parameters:  # sgd.py:343-347
+        if decouple_wd:
+            param.mul_(weight_decay)
+        else:
+            grad.add_(param, alpha=weight_decay)
+    if momentum != 0:  # sgd.py:349-357
+        if dampening:
+            exp_avg.lerp_(grad, weight=1 - momentum)
+        else:
+            exp_avg.mul_(momentum).add_(grad)
+    else:
+        exp_avg = grad
+    if not update_parameters:
+        return
+    if kahan_sum and param.dtype in LOW_PRECISION:  # sgd.py:360-369
+        kahan_comp.add_(exp_avg, alpha=-lr)
+        _kahan_commit(param, grad, kahan_comp)
+    else:  # sgd.py:372
+        param.add_(exp_avg, alpha=-lr)
+
+
+def sgd(params, grads, exp_avgs, kahan_comps=None, *, lr, momentum, weight_decay, dampening, decouple_wd,
+        decouple_lr=False, max_lr=None, kahan_sum=False, optimizer_accumulation=False, **_):
+    """Functional SGD step  (optimi/sgd.py:213-298)."""
+    if weight_decay != 0:  # sgd.py:256-260
+        if decouple_lr:
+            weight_decay = 1 - (lr / max_lr) * weight_decay
+        elif decouple_wd:
+            weight_decay = 1 - lr * weight_decay
+    params, grads, exp_avgs = map(_as_list, (params, grads, exp_avgs))
+    kahan_comps = [None] * len(params) if kahan_comps is None else _as_list(kahan_comps)
+    for p, g, m, k in zip(params, grads, exp_avgs, kahan_comps):
+        sgd_tensor(p, g, m, k, lr=lr, momentum=momentum, weight_decay=weight_decay, dampening=dampening,
+                   decouple_wd=(decouple_wd or decouple_lr), kahan_sum=kahan_sum,
+                   update_parameters=not optimizer_accumulation)
+
+
+# ----------------------------------------------------------------------------
+# RAdam and Ranger, one tensor          optimi/radam.py:368-417, ranger.py:402-473
+# ----------------------------------------------------------------------------
+def rectification(beta2: float, step: int):
+    """Variance rectification term, or None while the approximated SMA is too short
+    (optimi/radam.py:269-277, ranger.py:290-298)."""
+    rho_inf = 2 / (1 - beta2) - 1
+    rho = rho_inf - 2 * step * (beta2**step) / (1 - beta2**step)
+    if rho > 5:
+        return math.sqrt(((rho - 4) * (rho - 2) * rho_inf) / ((rho_inf - 4) * (rho_inf - 2) * rho))
+    return None
+
+
+def _radam_step(target, exp_avg, exp_avg_sq, *, lr, eps, rect):
+    """target += -lr*rect*m/(sqrt(v)+eps) once rectified, else -lr*m  (radam.py:398-417)."""
+    if rect is not None:
+        target.addcdiv_(exp_avg, exp_avg_sq.sqrt().add_(eps), value=-lr * rect)
+    else:
+        target.add_(exp_avg, alpha=-lr)
+
+
+def radam_tensor(param, grad, exp_avg, exp_avg_sq, kahan_comp, *, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay,
+                 eps, rect, decouple_wd, kahan_sum=False, update_parameters=True):
+    if weight_decay != 0 and update_parameters:  # radam.py:387-391
+        if decouple_wd:
+            param.mul_(weight_decay)
+        else:
+            grad.add_(param, alpha=weight_decay)
+    exp_avg.lerp_(grad, weight=beta1_comp)  # radam.py:394
+    exp_avg_sq.mul_(beta2_hat).addcmul_(grad, grad, value=beta2_comp)  # radam.py:395
+    if not update_parameters:
+        return
+    if kahan_sum and param.dtype in LOW_PRECISION:  # radam.py:398-410
+        _radam_step(kahan_comp, exp_avg, exp_avg_sq, lr=lr, eps=eps, rect=rect)
+        _kahan_commit(param, grad, kahan_comp)
+    else:  # radam.py:412-417
+        _radam_step(param, exp_avg, exp_avg_sq, lr=lr, eps=eps, rect=rect)
+
+
+def ranger_tensor(param, grad, exp_avg, exp_avg_sq, la_param, kahan_comp, *, lr, beta1_comp, beta2_hat, beta2_comp,
+                  weight_decay, eps, rect, k, alpha, step, decouple_wd, kahan_sum=False, update_parameters=True):
+    """RAdam step, then every ``k``-th step the Lookahead interpolation with the slow weights."""
+    radam_tensor(param, grad, exp_avg, exp_avg_sq, kahan_comp, lr=lr, beta1_comp=beta1_comp, beta2_hat=beta2_hat,
+                 beta2_comp=beta2_comp, weight_decay=weight_decay, eps=eps, rect=rect, decouple_wd=decouple_wd,
+                 kahan_sum=kahan_sum, update_parameters=update_parameters)
+    if not update_parameters or step % k != 0:
+        return
+    if kahan_sum and param.dtype in LOW_PRECISION:  # ranger.py:452-463
+        kahan_comp.add_(param.sub_(la_param), alpha=alpha)
+        grad.copy_(la_param.detach())
+        la_param.add_(kahan_comp)
+        kahan_comp.add_(grad.sub_(la_param), alpha=alpha)
+        param.copy_(la_param)
+    else:  # ranger.py:471-473
+        la_param.add_(param.sub(la_param), alpha=alpha)
+        param.copy_(la_param)
+
+
+def _radam_prologue(lr, beta1, beta2, weight_decay, step, decouple_wd, decouple_lr, max_lr):
+    t = _tick(step)
+    beta1_hat = debias_beta(beta1, t)
+    beta2_hat = debias_beta(beta2, t)
+    rect = rectification(beta2, t)
+    if weight_decay != 0:
+        if decouple_lr:
+            weight_decay = 1 - (lr / max_lr) * weight_decay
+        elif decouple_wd:
+            weight_decay = 1 - lr * weight_decay
+    return t, beta1_hat, beta2_hat, rect, weight_decay
+
+
+def radam(params, grads, exp_avgs, exp_avg_sqs, kahan_comps=None, *, lr, beta1, beta2, weight_decay, eps, step,
+          decouple_wd, decouple_lr=False, max_lr=None, kahan_sum=False, optimizer_accumulation=False, **_):
+    """Functional RAdam step  (optimi/radam.py:214-322)."""
+    _, b1h, b2h, rect, weight_decay = _radam_prologue(lr, beta1, beta2, weight_decay, step, decouple_wd, decouple_lr, max_lr)
+    params, grads, exp_avgs, exp_avg_sqs = map(_as_list, (params, grads, exp_avgs, exp_avg_sqs))
+    kahan_comps = [None] * len(params) if kahan_comps is None else _as_list(kahan_comps)
+    for p, g, m, v, kc in zip(params, grads, exp_avgs, exp_avg_sqs, kahan_comps):
+        radam_tensor(p, g, m, v, kc, lr=lr, beta1_comp=1 - b1h, beta2_hat=b2h, beta2_comp=1 - b2h,
+                     weight_decay=weight_decay, eps=eps, rect=rect, decouple_wd=(decouple_wd or decouple_lr),
+                     kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation)
+
+
+def ranger(params, grads, exp_avgs, exp_avg_sqs, la_params, kahan_comps=None, *, lr, beta1, beta2, weight_decay, eps,
+           k, alpha, step, decouple_wd, decouple_lr=False, max_lr=None, kahan_sum=False, optimizer_accumulation=False,
+           **_):
+    """Functional Ranger step  (optimi/ranger.py:230-344)."""
+    t, b1h, b2h, rect, weight_decay = _radam_prologue(lr, beta1, beta2, weight_decay, step, decouple_wd, decouple_lr, max_lr)
+    params, grads, exp_avgs, exp_avg_sqs, la_params = map(_as_list, (params, grads, exp_avgs, exp_avg_sqs, la_params))
+    kahan_comps = [None] * len(params) if kahan_comps is None else _as_list(kahan_comps)
+    for p, g, m, v, la, kc in zip(params, grads, exp_avgs, exp_avg_sqs, la_params, kahan_comps):
+        ranger_tensor(p, g, m, v, la, kc, lr=lr, beta1_comp=1 - b1h, beta2_hat=b2h, beta2_comp=1 - b2h,
+                      weight_decay=weight_decay, eps=eps, rect=rect, k=k, alpha=alpha, step=t,
+                      decouple_wd=(decouple_wd or decouple_lr), kahan_sum=kahan_sum,
+                      update_parameters=not optimizer_accumulation)
+
+
+# ----------------------------------------------------------------------------
 # A minimal stateful driver: what the reference's optimizer classes do around
 # the functional call (lazy state, step counters, Kahan tri-state), reduced to
 # plain lists so tests and the CPU baseline can run whole synthetic lists.
@@ -270,6 +417,9 @@ class ForLoopRun:
         "lion": dict(betas=(0.9, 0.99), weight_decay=0.0),
         "stableadamw": dict(betas=(0.9, 0.99), weight_decay=1e-2, eps=1e-6),
         "adan": dict(betas=(0.98, 0.92, 0.99), weight_decay=2e-2, eps=1e-6),
+        "sgd": dict(momentum=0.0, weight_decay=0.0, dampening=False, decouple_wd=False, torch_init=False),
+        "radam": dict(betas=(0.9, 0.99), weight_decay=0.0, eps=1e-6, decouple_wd=False),
+        "ranger": dict(betas=(0.9, 0.99), weight_decay=0.0, eps=1e-6, k=6, alpha=0.5, decouple_wd=True),
     }
 
     def __init__(self, name, params, *, gradient_release=False, **hyper):
@@ -293,8 +443,18 @@ class ForLoopRun:
             return self.state[i]
         p = self.params[i]
         st = {"exp_avg": torch.zeros_like(p)}
-        if self.name in ("adam", "adamw", "stableadamw", "adan"):
+        if self.name == "sgd":  # sgd.py:97-107
+            h = self.hyper
+            if h["dampening"] and h["torch_init"]:
+                st["exp_avg"] = grad.detach().clone()
+                if h["weight_decay"] != 0 and not h.get("decouple_lr") and not h["decouple_wd"]:
+                    st["exp_avg"].add_(p, alpha=h["weight_decay"])
+            elif h["momentum"] == 0:
+                st["exp_avg"] = None
+        if self.name in ("adam", "adamw", "stableadamw", "adan", "radam", "ranger"):
             st["exp_avg_sq"] = torch.zeros_like(p)
+        if self.name == "ranger":
+            st["la_param"] = p.detach().clone()  # ranger.py:142
         if self.name == "stableadamw":
             st["eps_sq"] = make_eps_sq(p, self.hyper["eps"])
         if self.name == "adan":
@@ -331,6 +491,17 @@ class ForLoopRun:
             h.pop("adam_wd", None)
             adan(ps, grads, col("exp_avg"), col("exp_avg_diff"), col("exp_avg_sq"), col("prev_grad"), col("kahan_comp"),
                  beta1=b1, beta2=b2, beta3=b3, **h, **common)
+        elif self.name == "sgd":
+            common.pop("step")
+            h.pop("torch_init", None)
+            sgd(ps, grads, col("exp_avg"), col("kahan_comp"), **h, **common)
+        elif self.name == "radam":
+            b1, b2 = h.pop("betas")
+            radam(ps, grads, col("exp_avg"), col("exp_avg_sq"), col("kahan_comp"), beta1=b1, beta2=b2, **h, **common)
+        elif self.name == "ranger":
+            b1, b2 = h.pop("betas")
+            ranger(ps, grads, col("exp_avg"), col("exp_avg_sq"), col("la_param"), col("kahan_comp"), beta1=b1, beta2=b2,
+                   **h, **common)
         else:
             raise ValueError(self.name)
 

@@ -10,6 +10,7 @@ raw CPU buffers to the C functions, so the two oracles share no arithmetic.
 from __future__ import annotations
 
 import ctypes as C
+import math
 import os
 import subprocess
 
@@ -21,7 +22,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "liboptimi_ref.so")
 
 F32, BF16 = 0, 1
-KAHAN, UPDATE, DECOUPLE_WD, ADAM_WD, DECOUPLE_LR = 1, 2, 4, 8, 16
+KAHAN, UPDATE, DECOUPLE_WD, ADAM_WD, DECOUPLE_LR, DAMPENING, RECTIFY, LOOKAHEAD = 1, 2, 4, 8, 16, 32, 64, 128
 
 _lib = None
 
@@ -45,6 +46,10 @@ def lib():
         L.optimi_ref_stableadamw.restype = d
         L.optimi_ref_adan.argtypes = [p, p, p, p, p, p, p, i64, i, d, d, d, d, d, d, d, d, i]
         L.optimi_ref_adan.restype = None
+        L.optimi_ref_sgd.argtypes = [p, p, p, p, i64, i, d, d, d, i]
+        L.optimi_ref_sgd.restype = None
+        L.optimi_ref_ranger.argtypes = [p, p, p, p, p, p, i64, i, d, d, d, d, d, d, d, d, i]
+        L.optimi_ref_ranger.restype = None
         _lib = L
     return _lib
 
@@ -92,7 +97,32 @@ def step_scalars(name: str, h: dict, t: int | None, kahan_sum: bool, accumulate:
         b1h, b2h, b3h = _beta_hat(b1, t), _beta_hat(b2, t), _beta_hat(b3, t)
         w = 1 + ratio * wd if wd != 0 else 0.0  # the class path is always Adan-style (adan.py:181-203)
         return (lr, 1 - b1h, b2, 1 - b2h, b3h, 1 - b3h, h["eps"], w, flags)
+    if name == "sgd":
+        decoupled = bool(h.get("decouple_wd") or h.get("decouple_lr"))
+        w = 1 - ratio * wd if (wd != 0 and decoupled) else wd
+        return (lr, h.get("momentum", 0.0), w,
+                flags | (DECOUPLE_WD if decoupled else 0) | (DAMPENING if h.get("dampening") else 0))
+    if name in ("radam", "ranger"):
+        b1, b2 = h.get("betas", (0.9, 0.99))
+        b1h, b2h = _beta_hat(b1, t), _beta_hat(b2, t)
+        decoupled = bool(h.get("decouple_wd") or h.get("decouple_lr"))
+        w = 1 - ratio * wd if (wd != 0 and decoupled) else wd
+        rect = rectification(b2, t)
+        f = flags | (DECOUPLE_WD if decoupled else 0) | (RECTIFY if rect is not None else 0)
+        if name == "ranger" and t % h.get("k", 6) == 0:
+            f |= LOOKAHEAD
+        head = (lr, 1 - b1h, b2h, 1 - b2h, w, h["eps"], rect if rect is not None else 0.0)
+        return head + ((h.get("alpha", 0.5), f) if name == "ranger" else (f,))
     raise ValueError(name)
+
+
+def rectification(beta2: float, t: int):
+    """RAdam's variance rectification term or None  (optimi/radam.py:269-277)."""
+    rho_inf = 2 / (1 - beta2) - 1
+    rho = rho_inf - 2 * t * (beta2**t) / (1 - beta2**t)
+    if rho > 5:
+        return math.sqrt(((rho - 4) * (rho - 2) * rho_inf) / ((rho_inf - 4) * (rho_inf - 2) * rho))
+    return None
 
 
 # state buffers each C entry point takes between ``grad`` and ``kahan_comp``
@@ -102,6 +132,9 @@ STATE_ORDER = {
     "lion": ("exp_avg",),
     "stableadamw": ("exp_avg", "exp_avg_sq"),
     "adan": ("exp_avg", "exp_avg_diff", "exp_avg_sq", "prev_grad"),
+    "sgd": ("exp_avg",),
+    "radam": ("exp_avg", "exp_avg_sq"),
+    "ranger": ("exp_avg", "exp_avg_sq", "la_param"),
 }
 
 
@@ -111,14 +144,19 @@ class ScalarRun(ForLoopRun):
     def _call(self, idxs, grads, step, accumulate):
         L = lib()
         t = None
-        if self.name != "lion":
+        if self.name not in ("lion", "sgd"):
             step.add_(1)
             t = int(step.item())
         scalars = step_scalars(self.name, self.hyper, t, self.kahan_sum, accumulate)
         fn = {"adam": L.optimi_ref_adam, "adamw": L.optimi_ref_adam, "lion": L.optimi_ref_lion,
-              "stableadamw": L.optimi_ref_stableadamw, "adan": L.optimi_ref_adan}[self.name]
+              "stableadamw": L.optimi_ref_stableadamw, "adan": L.optimi_ref_adan, "sgd": L.optimi_ref_sgd,
+              "radam": L.optimi_ref_ranger, "ranger": L.optimi_ref_ranger}[self.name]
         for i, g in zip(idxs, grads):
             st = self._ensure_state(i, g)
             p = self.params[i]
             bufs = [_ptr(st[k]) for k in STATE_ORDER[self.name]]
-            fn(_ptr(p), _ptr(g), *bufs, _ptr(st["kahan_comp"]), p.numel(), _dt(p), *scalars)
+            args = scalars
+            if self.name == "radam":  # the C function serves RAdam and Ranger: no slow weights, no alpha
+                bufs.append(None)
+                args = scalars[:-1] + (0.0, scalars[-1])
+            fn(_ptr(p), _ptr(g), *bufs, _ptr(st["kahan_comp"]), p.numel(), _dt(p), *args)

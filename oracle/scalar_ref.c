@@ -34,7 +34,10 @@ enum {
   OPTIMI_REF_UPDATE = 2,      /* update_parameters                                  */
   OPTIMI_REF_DECOUPLE_WD = 4, /* Adam: decoupled decay; unset = L2 into the gradient */
   OPTIMI_REF_ADAM_WD = 8,     /* Adan: Adam-style decay instead of Adan-style       */
-  OPTIMI_REF_DECOUPLE_LR = 16 /* StableAdamW: fully decoupled decay                 */
+  OPTIMI_REF_DECOUPLE_LR = 16,/* StableAdamW: fully decoupled decay                 */
+  OPTIMI_REF_DAMPENING = 32,  /* SGD: dampened momentum (lerp)                       */
+  OPTIMI_REF_RECTIFY = 64,    /* RAdam/Ranger: rectified step                        */
+  OPTIMI_REF_LOOKAHEAD = 128  /* Ranger: Lookahead sync on this step                 */
 };
 
 static inline float bits_to_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
@@ -253,6 +256,103 @@ void optimi_ref_adan(void* param, const void* grad, void* exp_avg, void* exp_avg
       p = R(p + (S(-lr * beta2) * df) / d, dt);                              /* adan.py:462 */
     }
     if (!adam_wd && weight_decay != 0) p = R(p / S(weight_decay), dt);       /* adan.py:465-466 */
+    ST(param, i, dt, p);
+  }
+}
+
+/* ---------------------------------------------------------------------------
+ * SGD                                                    optimi/sgd.py:329-372
+ * weight_decay as for Adam.  exp_avg may be NULL when momentum == 0.
+ * ------------------------------------------------------------------------- */
+void optimi_ref_sgd(void* param, const void* grad, void* exp_avg, void* kahan, int64_t n, int dt, double lr,
+                    double momentum, double weight_decay, int flags) {
+  const int update = (flags & OPTIMI_REF_UPDATE) != 0;
+  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && dt == OPTIMI_REF_BF16;
+  const int do_wd = weight_decay != 0 && update;
+  const float neg_lr = Sd(-lr, dt); /* add_(exp_avg, alpha=-lr) */
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float p = LD(param, i, dt), g = LD(grad, i, dt), m;
+    if (do_wd) {
+      if (flags & OPTIMI_REF_DECOUPLE_WD) p = R(p * S(weight_decay), dt);    /* sgd.py:345 */
+      else g = R(fmaf(p, Sd(weight_decay, dt), g), dt);                      /* sgd.py:347 */
+    }
+    if (momentum != 0) {
+      m = LD(exp_avg, i, dt);
+      if (flags & OPTIMI_REF_DAMPENING) {
+        m = R(lerp_f(m, g, S(1 - momentum)), dt);                            /* sgd.py:353 */
+      } else {
+        m = R(m * S(momentum), dt);                                          /* sgd.py:355 */
+        m = R(m + g, dt);
+      }
+      ST(exp_avg, i, dt, m);
+    } else {
+      m = g;                                                                 /* sgd.py:357 */
+    }
+    if (!update) continue;
+    if (do_kahan) {
+      float k = LD(kahan, i, dt);
+      k = R(fmaf(m, neg_lr, k), dt);                                         /* sgd.py:362 */
+      kahan_commit(&p, &k, dt);
+      ST(kahan, i, dt, k);
+    } else {
+      p = R(fmaf(m, neg_lr, p), dt);                                         /* sgd.py:372 */
+    }
+    ST(param, i, dt, p);
+  }
+}
+
+/* ---------------------------------------------------------------------------
+ * RAdam and Ranger                     optimi/radam.py:368-417, ranger.py:402-473
+ * rect is read only with OPTIMI_REF_RECTIFY.  la_param (Ranger) may be NULL for
+ * RAdam; with OPTIMI_REF_LOOKAHEAD the Lookahead interpolation follows the step.
+ * ------------------------------------------------------------------------- */
+void optimi_ref_ranger(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* la_param, void* kahan,
+                       int64_t n, int dt, double lr, double beta1_comp, double beta2_hat, double beta2_comp,
+                       double weight_decay, double eps, double rect, double alpha, int flags) {
+  const int update = (flags & OPTIMI_REF_UPDATE) != 0;
+  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && dt == OPTIMI_REF_BF16;
+  const int do_wd = weight_decay != 0 && update;
+  const int rectify = (flags & OPTIMI_REF_RECTIFY) != 0;
+  const int lookahead = update && (flags & OPTIMI_REF_LOOKAHEAD) && la_param;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float p = LD(param, i, dt), g = LD(grad, i, dt), m = LD(exp_avg, i, dt), v = LD(exp_avg_sq, i, dt);
+    if (do_wd) {
+      if (flags & OPTIMI_REF_DECOUPLE_WD) p = R(p * S(weight_decay), dt);    /* radam.py:389 */
+      else g = R(fmaf(p, Sd(weight_decay, dt), g), dt);                      /* radam.py:391 */
+    }
+    m = R(lerp_f(m, g, S(beta1_comp)), dt);                                  /* radam.py:394 */
+    v = R(v * S(beta2_hat), dt);                                             /* radam.py:395 */
+    v = R(fmaf(S(beta2_comp) * g, g, v), dt);
+    ST(exp_avg, i, dt, m);
+    ST(exp_avg_sq, i, dt, v);
+    if (!update) continue;
+    float k = do_kahan ? LD(kahan, i, dt) : p;   /* the accumulator the step lands in */
+    if (rectify) {
+      float d = R(sqrtf(v), dt);
+      d = R(d + Sd(eps, dt), dt);
+      k = R(k + (S(-lr * rect) * m) / d, dt);                                /* radam.py:401, 415 */
+    } else {
+      k = R(fmaf(m, Sd(-lr, dt), k), dt);                                    /* radam.py:403, 417 */
+    }
+    if (do_kahan) kahan_commit(&p, &k, dt); else p = k;
+    if (lookahead) {
+      float la = LD(la_param, i, dt);
+      float t = R(p - la, dt);                                               /* ranger.py:453, 472 */
+      if (do_kahan) {
+        k = R(fmaf(t, Sd(alpha, dt), k), dt);                                /* ranger.py:453 */
+        float old = la;
+        la = R(old + k, dt);                                                 /* ranger.py:457 */
+        float err = R(old - la, dt);
+        k = R(fmaf(err, Sd(alpha, dt), k), dt);                              /* ranger.py:460 */
+      } else {
+        la = R(fmaf(t, Sd(alpha, dt), la), dt);                              /* ranger.py:472 */
+      }
+      p = la;                                                                /* ranger.py:462, 473 */
+      ST(la_param, i, dt, la);
+    }
+    if (do_kahan) ST(kahan, i, dt, k);
     ST(param, i, dt, p);
   }
 }

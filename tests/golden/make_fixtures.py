@@ -2,7 +2,7 @@
 
 Run once, in a container that has the reference checkout, on CPU:
 
-    python tests/golden/make_fixtures.py [/root/reference]
+    python tests/golden/make_fixtures.py [/root/reference [case names...]]
 
 It imports optimi from that path, drives its optimizer classes with
 ``triton=False, foreach=False`` (the PyTorch for-loop path) on small seeded
@@ -34,6 +34,8 @@ ADAMW = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
 LION = dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1)
 SADAMW = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
 ADAN = dict(lr=1e-3, betas=(0.98, 0.92, 0.99), eps=1e-8, weight_decay=2e-2)
+SGD = dict(lr=1e-2, momentum=0.9, weight_decay=1e-2)
+RADAM = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
 
 # name -> (class name, kwargs, dtype, mode, n_steps)
 # mode "group": optimizer.step() on the whole list.
@@ -65,9 +67,35 @@ CASES = {
     "lion_bf16_kahan_release": ("Lion", dict(LION), "bfloat16", "release", 8),
     "stableadamw_bf16_kahan_release": ("StableAdamW", dict(SADAMW), "bfloat16", "release", 8),
     "adan_bf16_kahan_release": ("Adan", dict(ADAN, kahan_sum=True), "bfloat16", "release", 8),
+    # with beta2 = 0.99 RAdam/Ranger take the unrectified step for t <= 5 and the rectified one from t = 6
+    "sgd_fp32_l2": ("SGD", dict(SGD), "float32", "group", 10),
+    "sgd_fp32_nomomentum": ("SGD", dict(SGD, momentum=0.0, decouple_wd=True), "float32", "group", 10),
+    "sgd_bf16_kahan": ("SGD", dict(SGD, decouple_wd=True), "bfloat16", "group", 10),
+    "sgd_bf16_kahan_dampening": ("SGD", dict(SGD, dampening=True, torch_init=True), "bfloat16", "group", 10),
+    "sgd_bf16_plain_nomomentum": ("SGD", dict(SGD, momentum=0.0, kahan_sum=False), "bfloat16", "group", 10),
+    "sgd_bf16_kahan_release": ("SGD", dict(SGD, decouple_wd=True), "bfloat16", "release", 8),
+    "radam_fp32": ("RAdam", dict(RADAM, decouple_wd=True), "float32", "group", 10),
+    "radam_bf16_kahan": ("RAdam", dict(RADAM, decouple_wd=True), "bfloat16", "group", 10),
+    "radam_bf16_plain_l2": ("RAdam", dict(RADAM, kahan_sum=False), "bfloat16", "group", 10),
+    "radam_bf16_kahan_release": ("RAdam", dict(RADAM, decouple_wd=True), "bfloat16", "release", 8),
+    "ranger_fp32": ("Ranger", dict(RADAM), "float32", "group", 13),
+    "ranger_bf16_kahan": ("Ranger", dict(RADAM), "bfloat16", "group", 13),
+    "ranger_bf16_plain": ("Ranger", dict(RADAM, kahan_sum=False, k=3, alpha=0.8), "bfloat16", "group", 10),
+    "ranger_bf16_kahan_release": ("Ranger", dict(RADAM, k=4), "bfloat16", "release", 8),
 }
 
-STATE_KEYS = ("exp_avg", "exp_avg_sq", "exp_avg_diff", "prev_grad", "kahan_comp")
+# the first 25 cases keep the seeds they were generated with; later cases hash their name
+_FIRST_CASES = sorted(n for n in CASES if n.split("_")[0] in ("adam", "adamw", "lion", "stableadamw", "adan"))
+
+
+def case_seed(name: str) -> int:
+    if name in _FIRST_CASES:
+        return 1000 + _FIRST_CASES.index(name)
+    import zlib
+
+    return 2000 + zlib.crc32(name.encode()) % 100000
+
+STATE_KEYS = ("exp_avg", "exp_avg_sq", "exp_avg_diff", "prev_grad", "la_param", "kahan_comp")
 
 
 def to_np(t: torch.Tensor) -> np.ndarray:
@@ -146,8 +174,11 @@ def main():
     import optimi  # noqa: E402  (the reference; CPU for-loop path only)
 
     torch.set_num_threads(1)
-    for seed, name in enumerate(sorted(CASES)):
-        out = run_case(optimi, name, 1000 + seed)
+    only = set(sys.argv[2:])
+    for name in sorted(CASES):
+        if only and name not in only:
+            continue
+        out = run_case(optimi, name, case_seed(name))
         path = os.path.join(HERE, f"{name}.npz")
         np.savez_compressed(path, **out)
         print(f"{name}: {len(out)} arrays, {os.path.getsize(path) / 1024:.1f} KiB")

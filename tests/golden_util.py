@@ -25,7 +25,21 @@ CASES = _mk.CASES
 STATE_KEYS = _mk.STATE_KEYS
 N_TENSORS = len(_mk.SHAPES)
 
-OPT_NAME = {"Adam": "adam", "AdamW": "adamw", "Lion": "lion", "StableAdamW": "stableadamw", "Adan": "adan"}
+OPT_NAME = {"Adam": "adam", "AdamW": "adamw", "Lion": "lion", "StableAdamW": "stableadamw", "Adan": "adan",
+            "SGD": "sgd", "RAdam": "radam", "Ranger": "ranger"}
+
+
+def torch_tail(name: str, numel: int) -> int:
+    """How many trailing elements of a bf16 tensor of a fixture case to leave out when comparing
+    against anything but torch itself.  ATen's CPU ``add_(other, alpha=...)`` fuses
+    ``self + alpha*other`` in fp32 in its vector body but works in bf16 arithmetic (the product
+    rounded on its own) in the scalar loop over the last ``numel % 32`` elements, so the
+    reference's own output is not uniform there.  SGD (``p += -lr*m``), RAdam/Ranger before
+    rectification, Ranger's Lookahead and L2 weight decay go through that op; the kernels and
+    the C emulator follow the vector body everywhere."""
+    dtype = CASES[name][2]
+    uses_add_alpha = name.split("_")[0] in ("sgd", "radam", "ranger") or name.endswith("_l2")
+    return numel % 32 if (dtype == "bfloat16" and uses_add_alpha) else 0
 
 
 def case_names():
@@ -153,4 +167,5 @@ def compare_engines(got_eng, want_eng, what, exact: bool, body_only: int = 0):
             if exact:
                 assert_bits_equal(a, b, label)
             else:
-                assert_close_to_reference(a, b, label, param=q if key == "kahan_comp" else None, is_param=key == "param")
+                assert_close_to_reference(a, b, label, param=q if key == "kahan_comp" else None,
+                                          is_param=key in ("param", "la_param"))

@@ -30,13 +30,31 @@ class HipRun(ForLoopRun):
         self.group = cabi.Group()
         self.entry = "adam" if name == "adamw" else name
 
+    def _ensure_state(self, i, grad):
+        """A state that starts from arithmetic (SGD's ``torch_init`` momentum buffer) is built by the
+        oracle's own code on CPU copies and moved to the device, so that it starts from the CPU result;
+        every other state is zeros or a copy and is created on the device."""
+        arithmetic = self.name == "sgd" and self.hyper.get("dampening") and self.hyper.get("torch_init")
+        if self.state[i] is not None or not arithmetic:
+            return super()._ensure_state(i, grad)
+        p_dev = self.params[i]
+        self.params[i] = p_dev.detach().cpu()
+        try:
+            st = super()._ensure_state(i, grad.detach().cpu())
+        finally:
+            self.params[i] = p_dev
+        for k, v in st.items():
+            if torch.is_tensor(v) and k != "step":
+                st[k] = v.to(p_dev.device)
+        return st
+
     def _stream(self):
         return torch.cuda.current_stream().cuda_stream
 
     def _call(self, idxs, grads, step, accumulate):
         L = cabi.lib()
         t = None
-        if self.name != "lion":
+        if self.name not in ("lion", "sgd"):
             step.add_(1)
             t = int(step.item())
         scalars = step_scalars(self.name, self.hyper, t, self.kahan_sum, accumulate)

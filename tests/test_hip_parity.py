@@ -36,9 +36,17 @@ CONFIGS = {
     "stableadamw": dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2),
     "adan": dict(lr=1e-3, betas=(0.98, 0.92, 0.99), eps=1e-8, weight_decay=2e-2, kahan_sum=True),
     "adan_nowd": dict(lr=1e-3, betas=(0.98, 0.92, 0.99), eps=1e-8, weight_decay=0.0),
+    "sgd_momentum": dict(lr=1e-2, momentum=0.9, weight_decay=1e-2, decouple_wd=True),
+    "sgd_dampening_l2": dict(lr=1e-2, momentum=0.9, weight_decay=1e-2, dampening=True, torch_init=True),
+    "sgd_plain": dict(lr=1e-2, momentum=0.0, weight_decay=0.0),
+    "radam": dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2, decouple_wd=True),
+    "ranger": dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2, k=3, alpha=0.5),
 }
 OPT_OF = {"adamw": "adamw", "adam_l2": "adam", "adamw_declr": "adamw", "lion": "lion", "stableadamw": "stableadamw",
-          "adan": "adan", "adan_nowd": "adan"}
+          "adan": "adan", "adan_nowd": "adan", "sgd_momentum": "sgd", "sgd_dampening_l2": "sgd", "sgd_plain": "sgd",
+          "radam": "radam", "ranger": "ranger"}
+# configurations whose bf16 runs go through ATen's add_(x, alpha=...), which is not uniform over a tensor
+ADD_ALPHA = {"adam_l2", "sgd_momentum", "sgd_dampening_l2", "sgd_plain", "radam", "ranger"}
 
 
 def draw(sizes, dtype, steps, seed):
@@ -129,14 +137,14 @@ def test_random_lists_match_both_oracles(cfg, dtype, kahan, hip_device):
     guard.check()
     G.compare_engines(hip1, hip, f"{cfg} single-vs-multi", exact=True)
     G.compare_engines(hip, sca, f"{cfg} hip-vs-scalar", exact=name != "stableadamw")
-    # L2 decay on bf16: ATen's CPU add kernel runs `g + alpha * p` fused in fp32 in its vector body but
-    # in bf16 arithmetic (the product rounded on its own) in the scalar loop for the last numel % 32
-    # elements, so the reference differs from itself there.  The kernels follow the vector body.
-    tail = 32 if (cfg == "adam_l2" and dtype == torch.bfloat16) else 0
+    # bf16 add_(x, alpha=...): ATen's CPU kernel fuses `self + alpha * x` in fp32 in its vector body but
+    # works in bf16 arithmetic (the product rounded on its own) in the scalar loop for the last
+    # numel % 32 elements, so the reference differs from itself there.  The kernels follow the vector body.
+    tail = 32 if (cfg in ADD_ALPHA and dtype == torch.bfloat16) else 0
     G.compare_engines(hip, ref, f"{cfg} hip-vs-forloop", exact=False, body_only=tail)
 
 
-@pytest.mark.parametrize("cfg", ["adamw", "lion", "stableadamw", "adan"])
+@pytest.mark.parametrize("cfg", ["adamw", "lion", "stableadamw", "adan", "sgd_momentum", "radam", "ranger"])
 def test_unaligned_buffers(cfg, hip_device):
     """Views that start 2 bytes (bf16) past a 16-byte boundary take the element-wise path."""
     hyper, name = CONFIGS[cfg], OPT_OF[cfg]
@@ -154,7 +162,7 @@ def test_unaligned_buffers(cfg, hip_device):
     G.compare_engines(hip, sca, f"{cfg} unaligned", exact=name != "stableadamw")
 
 
-@pytest.mark.parametrize("cfg", ["adamw", "lion", "stableadamw", "adan"])
+@pytest.mark.parametrize("cfg", ["adamw", "lion", "stableadamw", "adan", "sgd_momentum", "radam", "ranger"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
 def test_gradient_release_with_accumulation(cfg, dtype, hip_device):
     """Per-tensor entry points in reverse order; 3 accumulate-only micro-steps, then a full one."""

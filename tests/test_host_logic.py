@@ -12,7 +12,10 @@ import optimi_amd
 from optimi_amd import functional as F
 from optimi_amd.utils import debias, debias_beta
 
-CLASSES = [optimi_amd.Adam, optimi_amd.AdamW, optimi_amd.Lion, optimi_amd.StableAdamW, optimi_amd.Adan]
+CLASSES = [optimi_amd.Adam, optimi_amd.AdamW, optimi_amd.Lion, optimi_amd.StableAdamW, optimi_amd.Adan,
+           optimi_amd.SGD, optimi_amd.RAdam, optimi_amd.Ranger]
+NO_BETAS = (optimi_amd.SGD,)
+NO_EPS = (optimi_amd.Lion, optimi_amd.SGD)
 
 
 def params():
@@ -25,11 +28,15 @@ def test_constructor_validation(cls):
         cls(params(), lr=-1.0)
     with pytest.raises(ValueError, match="weight decay"):
         cls(params(), lr=1e-3, weight_decay=-0.1)
-    with pytest.raises(ValueError, match="beta1"):
-        cls(params(), lr=1e-3, betas=(1.0, 0.9, 0.9)[: 3 if cls is optimi_amd.Adan else 2])
+    if cls not in NO_BETAS:
+        with pytest.raises(ValueError, match="beta1"):
+            cls(params(), lr=1e-3, betas=(1.0, 0.9, 0.9)[: 3 if cls is optimi_amd.Adan else 2])
+    else:
+        with pytest.raises(ValueError, match="momentum"):
+            cls(params(), lr=1e-3, momentum=1.0)
     with pytest.raises(ValueError, match="max_lr|maximum learning rate"):
         cls(params(), lr=1e-3, max_lr=-1.0)
-    if cls is not optimi_amd.Lion:
+    if cls not in NO_EPS:
         with pytest.raises(ValueError, match="epsilon"):
             cls(params(), lr=1e-3, eps=-1e-8)
     with pytest.raises(ValueError, match="foreach"):
@@ -46,10 +53,15 @@ def test_group_keys_and_decouple_lr_defaults(cls):
     assert any("potentially high for decouple_lr=True" in str(w.message) for w in caught)
     g = opt.param_groups[0]
     assert g["max_lr"] == 3e-4 and g["decouple_lr"] is True and g["setup"] is False
-    common = {"lr", "beta1", "beta2", "weight_decay", "decouple_lr", "max_lr", "kahan_sum", "foreach", "triton",
+    common = {"lr", "weight_decay", "decouple_lr", "max_lr", "kahan_sum", "foreach", "triton",
               "gradient_release", "setup", "params"}
-    extra = {optimi_amd.Adam: {"eps", "decouple_wd"}, optimi_amd.AdamW: {"eps", "decouple_wd"}, optimi_amd.Lion: set(),
-             optimi_amd.StableAdamW: {"eps"}, optimi_amd.Adan: {"eps", "beta3", "adam_wd"}}[cls]
+    betas = {"beta1", "beta2"}
+    extra = {optimi_amd.Adam: betas | {"eps", "decouple_wd"}, optimi_amd.AdamW: betas | {"eps", "decouple_wd"},
+             optimi_amd.Lion: betas, optimi_amd.StableAdamW: betas | {"eps"},
+             optimi_amd.Adan: betas | {"eps", "beta3", "adam_wd"},
+             optimi_amd.SGD: {"momentum", "dampening", "decouple_wd", "torch_init"},
+             optimi_amd.RAdam: betas | {"eps", "decouple_wd"},
+             optimi_amd.Ranger: betas | {"eps", "decouple_wd", "k", "alpha"}}[cls]
     assert {k for k in g if not k.startswith("_")} - {"params"} >= (common | extra) - {"params"}
     assert set(opt.state_dict()["param_groups"][0]) >= (common | extra)
     with warnings.catch_warnings():
@@ -102,6 +114,9 @@ def test_step_without_gradients_is_a_noop_that_still_counts():
     opt = optimi_amd.AdamW(ps, lr=1e-3)
     opt.step()
     assert int(opt.param_groups[0]["step"]) == 1 and len(opt.state) == 0
+    sgd = optimi_amd.SGD(params(), lr=1e-3)
+    sgd.step()
+    assert "step" not in sgd.param_groups[0]
 
 
 def test_gradient_release_setup_and_hooks():
