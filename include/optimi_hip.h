@@ -19,7 +19,7 @@
  *   - work is enqueued on `stream` (a hipStream_t; NULL = the default stream) and
  *     the call returns without waiting for it.
  *   - `kahan_comp` may be NULL whenever the Kahan branch is not taken (fp32 tensors,
- *     OPTIMI_KAHAN unset, or OPTIMI_UPDATE unset).
+ *     OPTIMI_KAHAN unset, or OPTIMI_UPDATE unset).  "Low precision" below means bf16 or fp16.
  *   - buffers aligned to 16 bytes take the vectorised path; any other alignment is
  *     accepted and runs an element-wise path.
  */
@@ -35,10 +35,10 @@ extern "C" {
 
 typedef void* optimi_stream_t; /* hipStream_t */
 
-enum optimi_dtype { OPTIMI_F32 = 0, OPTIMI_BF16 = 1 };
+enum optimi_dtype { OPTIMI_F32 = 0, OPTIMI_BF16 = 1, OPTIMI_F16 = 2 };
 
 enum optimi_flags {
-  OPTIMI_KAHAN = 1,       /* kahan_sum: only acts on bf16 tensors (optimi/adam.py:384)            */
+  OPTIMI_KAHAN = 1,       /* kahan_sum: only acts on bf16/fp16 tensors (optimi/adam.py:384)       */
   OPTIMI_UPDATE = 2,      /* update_parameters; unset = accumulate-only step (optimi/adam.py:308) */
   OPTIMI_DECOUPLE_WD = 4, /* Adam: decoupled decay p*=factor; unset = L2 (optimi/adam.py:373-377) */
   OPTIMI_ADAM_WD = 8,     /* Adan: Adam-style decay before the step (optimi/adan.py:447-448)      */

@@ -47,7 +47,7 @@ def default_group(device: torch.device, dtype: torch.dtype, tag: str = ""):
     return grp
 
 
-SUPPORTED_DTYPES = (torch.float32, torch.bfloat16)
+SUPPORTED_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
 
 
 def check_supported(param: torch.Tensor):
@@ -57,7 +57,7 @@ def check_supported(param: torch.Tensor):
             "There is no CPU path in this package."
         )
     if param.dtype not in SUPPORTED_DTYPES:
-        raise NotImplementedError(f"optimi_amd: parameter dtype {param.dtype} is not implemented (float32, bfloat16 are)")
+        raise NotImplementedError(f"optimi_amd: parameter dtype {param.dtype} is not implemented (float32, bfloat16 and float16 are)")
 
 
 def like_param(param: torch.Tensor, other: torch.Tensor) -> torch.Tensor:

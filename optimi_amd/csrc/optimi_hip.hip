@@ -52,6 +52,7 @@ constexpr int kAbiVersion = 1000;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 // Pointers come out of the tensor table as plain addresses; telling the compiler they are
 // global memory gets global_load/global_store instead of flat accesses.
@@ -112,6 +113,37 @@ struct BF16 {
   }
   __device__ static __forceinline__ void store1(void* p, int64_t i, float x) {
     ((OPTIMI_GLOBAL uint16_t*)(uintptr_t)p)[i] = (uint16_t)(__float_as_uint(x) >> 16);
+  }
+};
+
+struct F16 {
+  static constexpr int kVec = 8;
+  static constexpr int kPairs = 4;
+  static constexpr int kElemBytes = 2;
+  __device__ static __forceinline__ f32x2 widen(uint32_t two) {  // two packed halves -> two floats
+    return __builtin_convertvector(__builtin_bit_cast(f16x2, two), f32x2);
+  }
+  // Round to nearest even, subnormals kept.  The conversion is written as an instruction so that
+  // the compiler cannot merge it with the fma that feeds it: the merged form (v_fma_mixlo_f16)
+  // rounds the exact result once, while the reference rounds to fp32 first and to fp16 second.
+  __device__ static __forceinline__ uint32_t narrow(f32x2 x) {
+    uint32_t r;
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(x.x), "v"(x.y));
+    return r;
+  }
+  __device__ static __forceinline__ f32x2 R2(f32x2 x) { return widen(narrow(x)); }
+  __device__ static __forceinline__ void unpack(const u32x4& r, f32x2* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = widen(r[i]);
+  }
+  __device__ static __forceinline__ u32x4 pack(const f32x2* f) {
+    return u32x4{narrow(f[0]), narrow(f[1]), narrow(f[2]), narrow(f[3])};
+  }
+  __device__ static __forceinline__ float load1(const void* p, int64_t i) {
+    return (float)((const OPTIMI_GLOBAL _Float16*)(uintptr_t)p)[i];
+  }
+  __device__ static __forceinline__ void store1(void* p, int64_t i, float x) {
+    ((OPTIMI_GLOBAL uint16_t*)(uintptr_t)p)[i] = (uint16_t)narrow(f32x2{x, x});
   }
 };
 
@@ -647,7 +679,11 @@ inline float round_bf16_host(float f) {
   std::memcpy(&f, &u, 4);
   return f;
 }
-inline float Sd(double x, int dtype) { return dtype == OPTIMI_BF16 ? round_bf16_host((float)x) : (float)x; }
+inline float round_f16_host(float f) { return (float)(_Float16)f; }  // round-to-nearest-even, subnormals kept
+inline float Sd(double x, int dtype) {
+  return dtype == OPTIMI_BF16 ? round_bf16_host((float)x) : dtype == OPTIMI_F16 ? round_f16_host((float)x) : (float)x;
+}
+inline bool valid_dtype(int dtype) { return dtype == OPTIMI_F32 || dtype == OPTIMI_BF16 || dtype == OPTIMI_F16; }
 inline Lerp make_lerp(double weight) {
   float w = (float)weight;
   Lerp l;
@@ -655,8 +691,8 @@ inline Lerp make_lerp(double weight) {
   l.coef = l.small ? w : w - 1.0f;
   return l;
 }
-inline int64_t chunk_elems_rt(int dtype) { return dtype == OPTIMI_BF16 ? chunk_elems<BF16>() : chunk_elems<F32>(); }
-inline int elem_bytes(int dtype) { return dtype == OPTIMI_BF16 ? 2 : 4; }
+inline int64_t chunk_elems_rt(int dtype) { return dtype == OPTIMI_F32 ? chunk_elems<F32>() : chunk_elems<BF16>(); }
+inline int elem_bytes(int dtype) { return dtype == OPTIMI_F32 ? 4 : 2; }
 
 #define HIP_TRY(expr)                          \
   do {                                         \
@@ -742,7 +778,7 @@ int prepare_tables(optimi_group* g, int n_tensors, const void* const* const* lis
                    const int64_t* numel, int dtype, hipStream_t stream) {
   if (!g) return OPTIMI_ERR_NULL;
   if (n_tensors < 0) return OPTIMI_ERR_SIZE;
-  if (dtype != OPTIMI_F32 && dtype != OPTIMI_BF16) return OPTIMI_ERR_DTYPE;
+  if (!valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
   if (n_tensors > 0 && !numel) return OPTIMI_ERR_NULL;
   for (int a = 0; a < n_arrays; ++a)
     if ((need & bit(a)) && check_ptrs(n_tensors, lists[a])) return OPTIMI_ERR_NULL;
@@ -900,6 +936,10 @@ void dispatch(int dtype, bool kahan, bool update, int wd, Fn&& fn) {
     if (!update) fn(OpT<BF16, false, false, 0>{});
     else if (kahan) pick_wd(BF16{}, std::true_type{});
     else pick_wd(BF16{}, std::false_type{});
+  } else if (dtype == OPTIMI_F16) {
+    if (!update) fn(OpT<F16, false, false, 0>{});
+    else if (kahan) pick_wd(F16{}, std::true_type{});
+    else pick_wd(F16{}, std::false_type{});
   } else {
     if (!update) fn(OpT<F32, false, false, 0>{});
     else pick_wd(F32{}, std::false_type{});
@@ -922,6 +962,10 @@ void dispatch_tags(int dtype, bool kahan, bool update, int wd, Fn&& fn) {
     if (!update) fn(BF16{}, bool_c<false>{}, bool_c<false>{}, int_c<0>{});
     else if (kahan) pick_wd(BF16{}, bool_c<true>{});
     else pick_wd(BF16{}, bool_c<false>{});
+  } else if (dtype == OPTIMI_F16) {
+    if (!update) fn(F16{}, bool_c<false>{}, bool_c<false>{}, int_c<0>{});
+    else if (kahan) pick_wd(F16{}, bool_c<true>{});
+    else pick_wd(F16{}, bool_c<false>{});
   } else {
     if (!update) fn(F32{}, bool_c<false>{}, bool_c<false>{}, int_c<0>{});
     else pick_wd(F32{}, bool_c<false>{});
@@ -930,7 +974,7 @@ void dispatch_tags(int dtype, bool kahan, bool update, int wd, Fn&& fn) {
 
 int single_entry(TensorEntry& e, const void* const* ptrs, int n_arrays, uint32_t need, int64_t numel, int dtype) {
   if (numel < 0) return OPTIMI_ERR_SIZE;
-  if (dtype != OPTIMI_F32 && dtype != OPTIMI_BF16) return OPTIMI_ERR_DTYPE;
+  if (!valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
   if (numel > chunk_elems_rt(dtype) * ((int64_t)0x7fffffff / kSub)) return OPTIMI_ERR_SIZE;
   std::memset(&e, 0, sizeof(e));
   e.numel = numel;
@@ -1055,7 +1099,7 @@ StableP1Scalars stable_p1_scalars(int dtype, double beta1_comp, double beta2_hat
 }
 
 inline bool kahan_on(int dtype, uint32_t flags) {
-  return dtype == OPTIMI_BF16 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
+  return dtype != OPTIMI_F32 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
 }
 
 template <class DT>
@@ -1122,7 +1166,7 @@ const char* optimi_hip_error_string(int status) {
     case OPTIMI_OK: return "success";
     case OPTIMI_ERR_NULL: return "optimi_hip: a required pointer is NULL";
     case OPTIMI_ERR_SIZE: return "optimi_hip: negative or too large element/tensor count";
-    case OPTIMI_ERR_DTYPE: return "optimi_hip: unsupported dtype (expected OPTIMI_F32 or OPTIMI_BF16)";
+    case OPTIMI_ERR_DTYPE: return "optimi_hip: unsupported dtype (expected OPTIMI_F32, OPTIMI_BF16 or OPTIMI_F16)";
     case OPTIMI_ERR_ALIGN: return "optimi_hip: buffer not aligned to its element size";
     case OPTIMI_ERR_DEVICE: return "optimi_hip: group used on a different device than it was created on";
     case OPTIMI_ERR_NOMEM: return "optimi_hip: host allocation failed";
@@ -1136,7 +1180,7 @@ const char* optimi_hip_error_string(int status) {
 int optimi_hip_version(void) { return kAbiVersion; }
 
 int64_t optimi_hip_chunk_elems(int dtype) {
-  if (dtype != OPTIMI_F32 && dtype != OPTIMI_BF16) return OPTIMI_ERR_DTYPE;
+  if (!valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
   return chunk_elems_rt(dtype);
 }
 
@@ -1222,6 +1266,8 @@ int optimi_hip_stableadamw_multi(optimi_group* g, int n_tensors, void* const* pa
   std::memset(&none, 0, sizeof(none));
   rc = dtype == OPTIMI_BF16
            ? stable_run<BF16>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+       : dtype == OPTIMI_F16
+           ? stable_run<F16>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
            : stable_run<F32>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
   if (rc) return rc;
   return note_launch(g, stream);
@@ -1296,6 +1342,8 @@ int optimi_hip_stableadamw_single(optimi_group* g, void* param, const void* grad
   if (g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
   rc = dtype == OPTIMI_BF16
            ? stable_run<BF16>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+       : dtype == OPTIMI_F16
+           ? stable_run<F16>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
            : stable_run<F32>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
   if (rc) return rc;
   return note_launch(g, stream);

@@ -30,7 +30,8 @@ int dtype_code(const at::Tensor& t) {
   switch (t.scalar_type()) {
     case at::kFloat: return OPTIMI_F32;
     case at::kBFloat16: return OPTIMI_BF16;
-    default: TORCH_CHECK(false, "optimi_amd: unsupported parameter dtype ", t.scalar_type(), " (float32 and bfloat16 are implemented)");
+    case at::kHalf: return OPTIMI_F16;
+    default: TORCH_CHECK(false, "optimi_amd: unsupported parameter dtype ", t.scalar_type(), " (float32, bfloat16 and float16 are implemented)");
   }
   return -1;
 }
@@ -106,7 +107,7 @@ Prepared prepare(const TensorList& params, uint32_t flags) {
   Prepared pr;
   if (params.empty()) return pr;
   pr.dtype = dtype_code(params[0]);
-  pr.kahan = pr.dtype == OPTIMI_BF16 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
+  pr.kahan = pr.dtype != OPTIMI_F32 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
   pr.numel.reserve(params.size());
   pr.params.v.reserve(params.size());
   for (const at::Tensor& p : params) {
@@ -253,7 +254,7 @@ One prepare_one(const at::Tensor& p, const std::optional<at::Tensor>& kahan_comp
   check_param(p);
   One o;
   o.dtype = dtype_code(p);
-  o.kahan = o.dtype == OPTIMI_BF16 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
+  o.kahan = o.dtype != OPTIMI_F32 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
   if (o.kahan) {
     TORCH_CHECK(kahan_comp.has_value(), "optimi_amd: kahan_sum is on but the Kahan buffer is missing");
     check_like(p, *kahan_comp, "kahan_comp");

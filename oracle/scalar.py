@@ -21,7 +21,7 @@ from .forloop import ForLoopRun
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "liboptimi_ref.so")
 
-F32, BF16 = 0, 1
+F32, BF16, F16 = 0, 1, 2
 KAHAN, UPDATE, DECOUPLE_WD, ADAM_WD, DECOUPLE_LR, DAMPENING, RECTIFY, LOOKAHEAD = 1, 2, 4, 8, 16, 32, 64, 128
 
 _lib = None
@@ -46,6 +46,8 @@ def lib():
         L.optimi_ref_stableadamw.restype = d
         L.optimi_ref_adan.argtypes = [p, p, p, p, p, p, p, i64, i, d, d, d, d, d, d, d, d, i]
         L.optimi_ref_adan.restype = None
+        L.optimi_ref_round.argtypes = [C.c_float, i]
+        L.optimi_ref_round.restype = C.c_float
         L.optimi_ref_sgd.argtypes = [p, p, p, p, i64, i, d, d, d, i]
         L.optimi_ref_sgd.restype = None
         L.optimi_ref_ranger.argtypes = [p, p, p, p, p, p, i64, i, d, d, d, d, d, d, d, d, i]
@@ -56,7 +58,7 @@ def lib():
 
 def _dt(t: torch.Tensor) -> int:
     assert t.device.type == "cpu" and t.is_contiguous()
-    return {torch.float32: F32, torch.bfloat16: BF16}[t.dtype]
+    return {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}[t.dtype]
 
 
 def _ptr(t):

@@ -10,7 +10,7 @@
  * file spells that chain out one element at a time with every rounding point
  * written down:
  *
- *   R(x)    round fp32 x to the tensor dtype (bf16: round-to-nearest-even; fp32: x)
+ *   R(x)    round fp32 x to the tensor dtype (bf16, fp16: round-to-nearest-even; fp32: x)
  *   S(s)    a Python-double scalar narrowed to fp32 (mul_, lerp_, addcmul_, addcdiv_, div_)
  *   Sd(s)   a Python-double scalar narrowed to the tensor dtype (add_ with a scalar
  *           operand or an alpha: ATen's CPU add kernel casts both to the tensor dtype)
@@ -28,7 +28,7 @@
 #include <stdlib.h>
 #include <string.h>
 
-enum { OPTIMI_REF_F32 = 0, OPTIMI_REF_BF16 = 1 };
+enum { OPTIMI_REF_F32 = 0, OPTIMI_REF_BF16 = 1, OPTIMI_REF_F16 = 2 };
 enum {
   OPTIMI_REF_KAHAN = 1,       /* kahan_sum requested (only acts on bf16 tensors)   */
   OPTIMI_REF_UPDATE = 2,      /* update_parameters                                  */
@@ -49,15 +49,53 @@ static inline uint16_t bf16_from_f32(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);
   return (uint16_t)(u >> 16);
 }
+/* IEEE binary16, round-to-nearest-even, subnormals kept, overflow to infinity */
+static inline uint16_t f16_from_f32(float f) {
+  const uint32_t inf32 = 255u << 23, max16 = (127u + 16u) << 23, magic = ((127u - 15u) + (23u - 10u) + 1u) << 23;
+  uint32_t u = f32_to_bits(f);
+  const uint32_t sign = u & 0x80000000u;
+  u ^= sign;
+  uint16_t o;
+  if (u >= max16) {
+    o = u > inf32 ? 0x7e00 : 0x7c00;
+  } else if (u < (113u << 23)) { /* below 2^-14: lands on the subnormal grid by adding a float whose ulp is 2^-24 */
+    float t = bits_to_f32(u) + bits_to_f32(magic);
+    o = (uint16_t)(f32_to_bits(t) - magic);
+  } else {
+    const uint32_t odd = (u >> 13) & 1u;
+    u += ((uint32_t)(15 - 127) << 23) + 0xfffu + odd;
+    o = (uint16_t)(u >> 13);
+  }
+  return (uint16_t)(o | (sign >> 16));
+}
+static inline float f16_to_f32(uint16_t h) {
+  const uint32_t sign = ((uint32_t)h & 0x8000u) << 16, ex = (h >> 10) & 0x1fu, man = h & 0x3ffu;
+  if (ex == 0) {
+    float v = (float)man * 5.9604644775390625e-8f; /* man * 2^-24 */
+    return sign ? -v : v;
+  }
+  if (ex == 31) return bits_to_f32(sign | 0x7f800000u | (man << 13));
+  return bits_to_f32(sign | ((ex + 112u) << 23) | (man << 13));
+}
+static inline int low_precision(int dt) { return dt != OPTIMI_REF_F32; }
 static inline float R(float x, int dt) {
-  return dt == OPTIMI_REF_BF16 ? bits_to_f32((uint32_t)bf16_from_f32(x) << 16) : x;
+  if (dt == OPTIMI_REF_BF16) return bits_to_f32((uint32_t)bf16_from_f32(x) << 16);
+  if (dt == OPTIMI_REF_F16) return f16_to_f32(f16_from_f32(x));
+  return x;
 }
 static inline float LD(const void* a, int64_t i, int dt) {
-  return dt == OPTIMI_REF_BF16 ? bits_to_f32((uint32_t)((const uint16_t*)a)[i] << 16) : ((const float*)a)[i];
+  if (dt == OPTIMI_REF_BF16) return bits_to_f32((uint32_t)((const uint16_t*)a)[i] << 16);
+  if (dt == OPTIMI_REF_F16) return f16_to_f32(((const uint16_t*)a)[i]);
+  return ((const float*)a)[i];
 }
 static inline void ST(void* a, int64_t i, int dt, float x) {
-  if (dt == OPTIMI_REF_BF16) ((uint16_t*)a)[i] = bf16_from_f32(x); else ((float*)a)[i] = x;
+  if (dt == OPTIMI_REF_BF16) ((uint16_t*)a)[i] = bf16_from_f32(x);
+  else if (dt == OPTIMI_REF_F16) ((uint16_t*)a)[i] = f16_from_f32(x);
+  else ((float*)a)[i] = x;
 }
+/* test hook: R() as the emulator applies it */
+float optimi_ref_round(float x, int dt) { return R(x, dt); }
+
 static inline float S(double s) { return (float)s; }
 static inline float Sd(double s, int dt) { return R((float)s, dt); }
 
@@ -83,7 +121,7 @@ void optimi_ref_adam(void* param, const void* grad, void* exp_avg, void* exp_avg
                      double lr, double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay,
                      double eps, int flags) {
   const int update = (flags & OPTIMI_REF_UPDATE) != 0;
-  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && dt == OPTIMI_REF_BF16;
+  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && low_precision(dt);
   const int do_wd = weight_decay != 0 && update;
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < n; ++i) {
@@ -119,7 +157,7 @@ void optimi_ref_adam(void* param, const void* grad, void* exp_avg, void* exp_avg
 void optimi_ref_lion(void* param, const void* grad, void* exp_avg, void* kahan, int64_t n, int dt, double lr,
                      double beta1_comp, double beta2_comp, double weight_decay, int flags) {
   const int update = (flags & OPTIMI_REF_UPDATE) != 0;
-  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && dt == OPTIMI_REF_BF16;
+  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && low_precision(dt);
   const int do_wd = weight_decay != 0 && update;
   const float neg_lr = Sd(-lr, dt); /* add_(update, alpha=-lr): alpha takes the tensor dtype */
 #pragma omp parallel for schedule(static)
@@ -157,7 +195,7 @@ double optimi_ref_stableadamw(void* param, const void* grad, void* exp_avg, void
                               int dt, double lr, double beta1_comp, double beta2_hat, double beta2_comp,
                               double weight_decay, double eps, double max_lr, int flags) {
   const int update = (flags & OPTIMI_REF_UPDATE) != 0;
-  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && dt == OPTIMI_REF_BF16;
+  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && low_precision(dt);
   const float eps_sq = R((float)(eps * eps), dt);                 /* stableadamw.py:119 */
   enum { BLK = 4096 };
   const int64_t nblk = (n + BLK - 1) / BLK;
@@ -223,7 +261,7 @@ void optimi_ref_adan(void* param, const void* grad, void* exp_avg, void* exp_avg
                      double beta2_comp, double beta3_hat, double beta3_comp, double eps, double weight_decay,
                      int flags) {
   const int update = (flags & OPTIMI_REF_UPDATE) != 0;
-  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && dt == OPTIMI_REF_BF16;
+  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && low_precision(dt);
   const int adam_wd = (flags & OPTIMI_REF_ADAM_WD) != 0;
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < n; ++i) {
@@ -267,7 +305,7 @@ void optimi_ref_adan(void* param, const void* grad, void* exp_avg, void* exp_avg
 void optimi_ref_sgd(void* param, const void* grad, void* exp_avg, void* kahan, int64_t n, int dt, double lr,
                     double momentum, double weight_decay, int flags) {
   const int update = (flags & OPTIMI_REF_UPDATE) != 0;
-  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && dt == OPTIMI_REF_BF16;
+  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && low_precision(dt);
   const int do_wd = weight_decay != 0 && update;
   const float neg_lr = Sd(-lr, dt); /* add_(exp_avg, alpha=-lr) */
 #pragma omp parallel for schedule(static)
@@ -311,7 +349,7 @@ void optimi_ref_ranger(void* param, const void* grad, void* exp_avg, void* exp_a
                        int64_t n, int dt, double lr, double beta1_comp, double beta2_hat, double beta2_comp,
                        double weight_decay, double eps, double rect, double alpha, int flags) {
   const int update = (flags & OPTIMI_REF_UPDATE) != 0;
-  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && dt == OPTIMI_REF_BF16;
+  const int do_kahan = (flags & OPTIMI_REF_KAHAN) && low_precision(dt);
   const int do_wd = weight_decay != 0 && update;
   const int rectify = (flags & OPTIMI_REF_RECTIFY) != 0;
   const int lookahead = update && (flags & OPTIMI_REF_LOOKAHEAD) && la_param;

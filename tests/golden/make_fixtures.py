@@ -8,7 +8,7 @@ It imports optimi from that path, drives its optimizer classes with
 ``triton=False, foreach=False`` (the PyTorch for-loop path) on small seeded
 tensors, and stores inputs (initial params, the gradient of every step) and
 outputs (params and every state tensor after selected steps) as ``.npz``
-files.  bf16 tensors are stored as their raw 16-bit patterns (uint16).
+files.  bf16 tensors are stored as their raw 16-bit patterns (uint16), fp16 as numpy float16.
 
 The fixtures are data only; the tests read them with ``numpy.load`` and never
 need the reference.  Each case is described in ``CASES`` below, which the tests
@@ -82,6 +82,17 @@ CASES = {
     "ranger_bf16_kahan": ("Ranger", dict(RADAM), "bfloat16", "group", 13),
     "ranger_bf16_plain": ("Ranger", dict(RADAM, kahan_sum=False, k=3, alpha=0.8), "bfloat16", "group", 10),
     "ranger_bf16_kahan_release": ("Ranger", dict(RADAM, k=4), "bfloat16", "release", 8),
+    # fp16: gradients of std 1e-3 square into fp16's subnormal range, which the states must round into
+    "adamw_fp16_kahan": ("AdamW", dict(ADAMW), "float16", "group", 10),
+    "adamw_fp16_kahan_release": ("AdamW", dict(ADAMW), "float16", "release", 8),
+    "lion_fp16_kahan": ("Lion", dict(LION), "float16", "group", 10),
+    "stableadamw_fp16_kahan": ("StableAdamW", dict(SADAMW), "float16", "group", 10),
+    # eps 1e-8 is 0 in fp16: where exp_avg_sq underflows to 0 as well the reference divides 0 by 0,
+    # and those elements are NaN from the first step on; the kernels must produce NaN in the same places
+    "adan_fp16_kahan": ("Adan", dict(ADAN, kahan_sum=True), "float16", "group", 10),
+    "adan_fp16_kahan_eps1e-6": ("Adan", dict(ADAN, kahan_sum=True, eps=1e-6), "float16", "group", 10),
+    "sgd_fp16_kahan": ("SGD", dict(SGD, decouple_wd=True), "float16", "group", 10),
+    "ranger_fp16_plain": ("Ranger", dict(RADAM, kahan_sum=False, k=3), "float16", "group", 10),
 }
 
 # the first 25 cases keep the seeds they were generated with; later cases hash their name
@@ -102,7 +113,7 @@ def to_np(t: torch.Tensor) -> np.ndarray:
     t = t.detach().cpu().contiguous()
     if t.dtype == torch.bfloat16:
         return t.view(torch.int16).numpy().view(np.uint16).copy()
-    return t.numpy().copy()
+    return t.numpy().copy()  # float16 is stored as numpy float16, bf16 as raw uint16
 
 
 def grad_scale(step: int) -> float:

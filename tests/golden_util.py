@@ -39,7 +39,7 @@ def torch_tail(name: str, numel: int) -> int:
     the C emulator follow the vector body everywhere."""
     dtype = CASES[name][2]
     uses_add_alpha = name.split("_")[0] in ("sgd", "radam", "ranger") or name.endswith("_l2")
-    return numel % 32 if (dtype == "bfloat16" and uses_add_alpha) else 0
+    return numel % 32 if (dtype in ("bfloat16", "float16") and uses_add_alpha) else 0
 
 
 def case_names():
@@ -94,10 +94,11 @@ def replay(name: str, fx: dict, make_engine, device="cpu") -> dict[str, torch.Te
 # comparison helpers
 # ----------------------------------------------------------------------------
 def bf16_ordinal(t: torch.Tensor) -> torch.Tensor:
-    """Maps bf16 values to integers so that adjacent representable values differ by 1."""
+    """Maps bf16 (or fp16) values to integers so that adjacent representable values differ by 1."""
     bits = t.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
     neg = bits >= 0x8000
-    return torch.where(neg, 0x8000 - bits, bits)
+    # every NaN maps to one ordinal: its sign and payload are not part of the result
+    return torch.where(torch.isnan(t), torch.full_like(bits, 1 << 20), torch.where(neg, 0x8000 - bits, bits))
 
 
 def bf16_ulp_diff(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
@@ -105,7 +106,10 @@ def bf16_ulp_diff(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 
 def bf16_ulp_of(t: torch.Tensor) -> torch.Tensor:
-    """Size of one bf16 ulp at each value of ``t`` (as fp32)."""
+    """Size of one ulp of ``t``'s dtype (bf16 or fp16) at each value of ``t`` (as fp32)."""
+    if t.dtype == torch.float16:
+        f = t.float().abs().clamp_min(2.0**-14)  # subnormals share the ulp of the smallest normal
+        return torch.exp2(torch.floor(torch.log2(f)) - 10)
     f = t.float().abs().clamp_min(2.0**-126)
     return torch.exp2(torch.floor(torch.log2(f)) - 7)
 
@@ -119,8 +123,8 @@ def fp32_rel_err(a: torch.Tensor, b: torch.Tensor, floor: float) -> torch.Tensor
 def assert_bits_equal(got: torch.Tensor, want: torch.Tensor, what: str):
     a = got.detach().cpu().contiguous()
     b = want.detach().cpu().contiguous()
-    view = torch.int16 if a.dtype == torch.bfloat16 else torch.int32
-    bad = a.view(view) != b.view(view)
+    view = torch.int16 if a.dtype in (torch.bfloat16, torch.float16) else torch.int32
+    bad = (a.view(view) != b.view(view)) & ~(torch.isnan(a) & torch.isnan(b))  # a NaN's sign and payload are free
     assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} elements differ (first at {int(bad.flatten().nonzero()[0])})"
 
 
@@ -131,7 +135,19 @@ def assert_close_to_reference(got, want, what, *, param=None, is_param=False):
     judged against the size of those terms - 1e-2 for parameters (the distance ten steps can move
     a parameter at lr 1e-3; i.e. |a-b| <= 1e-8 near zero) and the tensor's RMS for moment states."""
     got, want = got.detach().cpu(), want.detach().cpu()
-    if want.dtype == torch.bfloat16:
+    # overflow and 0/0 must happen in the same places with the same outcome (fp16 reaches both);
+    # the tolerance below then applies to the finite elements
+    wild = ~torch.isfinite(want)
+    if bool(wild.any()) or not bool(torch.isfinite(got).all()):
+        assert torch.equal(torch.isnan(got), torch.isnan(want)), f"{what}: NaN in different places"
+        inf = torch.isinf(want)
+        assert torch.equal(torch.isinf(got), inf) and torch.equal(got[inf], want[inf]), f"{what}: inf in different places"
+        got, want = got.masked_fill(wild, 0), want.masked_fill(wild, 0)
+        if param is not None:
+            param = param.detach().cpu()
+            got, want = got.masked_fill(~torch.isfinite(param), 0), want.masked_fill(~torch.isfinite(param), 0)
+            param = param.masked_fill(~torch.isfinite(param), 1)
+    if want.dtype in (torch.bfloat16, torch.float16):
         if param is not None:
             err = (got.float() - want.float()).abs() / bf16_ulp_of(param.detach().cpu())
             assert float(err.max()) <= 1.0, f"{what}: Kahan buffer off by {float(err.max()):.3f} parameter ulps"

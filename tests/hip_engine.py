@@ -14,7 +14,7 @@ from optimi_amd import cabi
 from oracle.forloop import ForLoopRun
 from oracle.scalar import STATE_ORDER, step_scalars
 
-DT = {torch.float32: cabi.F32, torch.bfloat16: cabi.BF16}
+DT = {torch.float32: cabi.F32, torch.bfloat16: cabi.BF16, torch.float16: cabi.F16}
 
 
 def _addr(t):

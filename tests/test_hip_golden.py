@@ -33,7 +33,7 @@ def compare_snapshot(name, key, got, want, param_want=None):
     got, want = got.flatten()[:keep], want.flatten()[:keep]
     if param_want is not None:
         param_want = param_want.flatten()[:keep]
-    if want.dtype == torch.bfloat16:
+    if want.dtype in (torch.bfloat16, torch.float16):
         ulp = G.bf16_ulp_diff(got, want)
         if "stableadamw" not in name:
             assert int(ulp.max()) == 0, f"{name} {key}: {int((ulp > 0).sum())} of {ulp.numel()} differ, max {int(ulp.max())} ulp"

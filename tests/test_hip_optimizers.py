@@ -67,7 +67,7 @@ def oracle_for(oname, params, hyper, **kw):
 def compare(opt, params, ref, what):
     # bf16 SGD / RAdam / Ranger: the reference is not uniform over the last numel % 32 elements
     # (scalar remainder loop of ATen's add_(x, alpha=...)); those are left out
-    cut = ref.name in ("sgd", "radam", "ranger") and params[0].dtype == torch.bfloat16
+    cut = ref.name in ("sgd", "radam", "ranger") and params[0].dtype != torch.float32
     for i, p in enumerate(params):
         keep = p.numel() - (p.numel() % 32 if cut else 0)
         if keep == 0:
@@ -84,7 +84,7 @@ def compare(opt, params, ref, what):
                                         is_param=key == "la_param")
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16], ids=["bf16", "fp32", "fp16"])
 @pytest.mark.parametrize("case", list(CASES))
 def test_normal_with_state_dict_roundtrip(case, dtype, hip_device):
     cls, oname, hyper = CASES[case]

@@ -113,8 +113,9 @@ def hip_engine(name, params, device, guard, offset=0, **kw):
     return eng
 
 
-@pytest.mark.parametrize("dtype,kahan", [(torch.bfloat16, None), (torch.bfloat16, False), (torch.float32, None)],
-                         ids=["bf16_kahan", "bf16_plain", "fp32"])
+@pytest.mark.parametrize("dtype,kahan", [(torch.bfloat16, None), (torch.bfloat16, False), (torch.float32, None),
+                                         (torch.float16, None), (torch.float16, False)],
+                         ids=["bf16_kahan", "bf16_plain", "fp32", "fp16_kahan", "fp16_plain"])
 @pytest.mark.parametrize("cfg", list(CONFIGS))
 def test_random_lists_match_both_oracles(cfg, dtype, kahan, hip_device):
     hyper = dict(CONFIGS[cfg])
@@ -140,7 +141,7 @@ def test_random_lists_match_both_oracles(cfg, dtype, kahan, hip_device):
     # bf16 add_(x, alpha=...): ATen's CPU kernel fuses `self + alpha * x` in fp32 in its vector body but
     # works in bf16 arithmetic (the product rounded on its own) in the scalar loop for the last
     # numel % 32 elements, so the reference differs from itself there.  The kernels follow the vector body.
-    tail = 32 if (cfg in ADD_ALPHA and dtype == torch.bfloat16) else 0
+    tail = 32 if (cfg in ADD_ALPHA and dtype != torch.float32) else 0
     G.compare_engines(hip, ref, f"{cfg} hip-vs-forloop", exact=False, body_only=tail)
 
 
@@ -163,7 +164,7 @@ def test_unaligned_buffers(cfg, hip_device):
 
 
 @pytest.mark.parametrize("cfg", ["adamw", "lion", "stableadamw", "adan", "sgd_momentum", "radam", "ranger"])
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16], ids=["bf16", "fp32", "fp16"])
 def test_gradient_release_with_accumulation(cfg, dtype, hip_device):
     """Per-tensor entry points in reverse order; 3 accumulate-only micro-steps, then a full one."""
     hyper, name = CONFIGS[cfg], OPT_OF[cfg]

@@ -222,3 +222,30 @@ def test_kahan_flag_is_ignored_for_fp32(engine):
     b = run(engine, "adamw", params, grads, kahan_sum=False, **hyper)
     for i in range(len(params)):
         assert torch.equal(a.params[i], b.params[i])
+
+
+def test_emulator_rounding_matches_numpy_and_torch():
+    """The C emulator's own fp16 / bf16 conversions (round to nearest even, fp16 subnormals,
+    overflow to inf) against numpy's float16 and torch's bfloat16 casts."""
+    from oracle import scalar
+
+    L = scalar.lib()
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([
+        rng.normal(size=20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, size=20000).astype(np.float32),
+        np.arange(0, 1 << 16, dtype=np.uint16).view(np.float16).astype(np.float32),  # every fp16 value
+        # ties between neighbouring fp16 values, normal and subnormal
+        (np.arange(0, 1 << 15, 97, dtype=np.uint16).view(np.float16).astype(np.float64)
+         + np.arange(1, (1 << 15) + 1, 97, dtype=np.uint16).view(np.float16).astype(np.float64)).astype(np.float32) / 2,
+        np.array([65504.0, 65519.9, 65520.0, 1e6, -1e6, 2.0**-25, 2.0**-25 * 1.0001, 2.0**-24, 0.0, -0.0], dtype=np.float32),
+    ])
+    xs = xs[np.isfinite(xs)]
+    with np.errstate(over="ignore"):
+        want16 = xs.astype(np.float16).astype(np.float32)
+    wantbf = torch.from_numpy(xs).to(torch.bfloat16).float().numpy()
+    got16 = np.array([L.optimi_ref_round(float(x), scalar.F16) for x in xs], dtype=np.float32)
+    gotbf = np.array([L.optimi_ref_round(float(x), scalar.BF16) for x in xs], dtype=np.float32)
+    got32 = np.array([L.optimi_ref_round(float(x), scalar.F32) for x in xs], dtype=np.float32)
+    assert np.array_equal(got16.view(np.uint32), want16.view(np.uint32))
+    assert np.array_equal(gotbf.view(np.uint32), wantbf.view(np.uint32))
+    assert np.array_equal(got32.view(np.uint32), xs.view(np.uint32))
