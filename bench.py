@@ -54,6 +54,13 @@ def workloads():
         "stableadamw_bf16_kahan_llama7b": ("StableAdamW", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2), "bfloat16", l7, 22),
         "adan_bf16_kahan_llama7b": ("Adan", dict(lr=1e-3, betas=(0.98, 0.92, 0.99), eps=1e-8, weight_decay=2e-2, kahan_sum=True), "bfloat16", l7, 26),
         "adamw_fp32_mlp": ("AdamW", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2), "float32", mlp, 28),
+        "adamw_fp32_llama1b": ("AdamW", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2), "float32", l1, 28),
+        "adamw_fp16_kahan_llama7b": ("AdamW", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2), "float16", l7, 18),
+        # p, g, exp_avg, kahan_comp read; p, exp_avg, kahan_comp written
+        "sgd_bf16_kahan_llama7b": ("SGD", dict(lr=1e-2, momentum=0.9, weight_decay=1e-2, decouple_wd=True), "bfloat16", l7, 14),
+        "radam_bf16_kahan_llama7b": ("RAdam", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2, decouple_wd=True), "bfloat16", l7, 18),
+        # as Adam; every k-th step also reads and writes the slow weights (4 more bytes per param on that step)
+        "ranger_bf16_kahan_llama7b": ("Ranger", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2, k=6, alpha=0.5), "bfloat16", l7, 18),
     }
 
 
@@ -98,7 +105,7 @@ def cpu_baseline(cls_name, kwargs, dtype, shapes, budget_s=20.0):
     sample = shapes if total <= 64_000_000 else shapes[1:10]
     what = "whole list" if sample is shapes else "one transformer layer (tensors 1-9 of the list)"
     n = sum(numel(s) for s in sample)
-    name = {"AdamW": "adamw", "Adam": "adam", "Lion": "lion", "StableAdamW": "stableadamw", "Adan": "adan"}[cls_name]
+    name = cls_name.lower()
     params = make_tensors(sample, dtype, "cpu", 1, 0.02, ones_for_1d=True)
     grads = make_tensors(sample, dtype, "cpu", 2, 1e-3)
     run = ForLoopRun(name, params, **kwargs)
@@ -187,6 +194,10 @@ def main():
     kernel_ms = [a.elapsed_time(b) for a, b in zip(starts, stops)]
     mean_kernel_ms = sum(kernel_ms) / len(kernel_ms)
 
+    if cls_name == "Ranger":  # average over the timed steps, of which every k-th is a Lookahead step
+        k = kwargs["k"]
+        slow = sum(1 for t in range(args.warmup + 1, args.warmup + args.steps + 1) if t % k == 0)
+        bytes_per_param += 4.0 * slow / args.steps
     algo_bytes = bytes_per_param * n_params
     achieved = algo_bytes / (mean_kernel_ms * 1e-3) / 1e9
     traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
@@ -201,7 +212,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if dtype == torch.bfloat16 else "f32",
+        "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype],
         "data": "synthetic",
         "config": {"workload": args.workload, "optimizer": cls_name, "n_tensors": len(shapes), "n_params": n_params,
                    "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()},
