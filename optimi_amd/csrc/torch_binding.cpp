@@ -12,7 +12,9 @@
 #include <torch/extension.h>
 
 #include <cmath>
+#include <cstring>
 #include <optional>
+#include <unordered_set>
 #include <vector>
 
 #include "optimi_hip.h"
@@ -320,87 +322,6 @@ void adan_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, 
 }
 
 
-// ---- gradient-release fast path --------------------------------------------------------
-// One call per parameter from the post-accumulate-grad hook: advances the parameter's int32
-// CPU step counter, forms the step scalars in double exactly as the functional forms do in
-// Python (optimi/adam.py:260-273, lion.py:226-235, stableadamw.py:326-332, adan.py:289-309)
-// and launches the per-tensor kernel.  std::pow(double, double) is libm's pow, the function
-// CPython's float ** int ends in, so the scalars are bit-identical to the Python path.
-
-double debias_beta(double beta, int64_t step) {  // optimi/utils.py:31-36
-  const double bt = std::pow(beta, (double)step);
-  return (bt - beta) / (bt - 1.0);
-}
-
-int64_t tick(const at::Tensor& step) {
-  TORCH_CHECK(step.device().is_cpu() && step.scalar_type() == at::kInt && step.numel() == 1,
-              "optimi_amd: the step counter must be a one-element int32 CPU tensor");
-  int32_t* s = step.data_ptr<int32_t>();
-  *s += 1;
-  return *s;
-}
-
-// The Kahan buffer if it is one: placeholders (one element, maybe another dtype) and None count as absent.
-std::optional<at::Tensor> real_kahan(const at::Tensor& p, const std::optional<at::Tensor>& k) {
-  if (!k.has_value() || !k->defined() || k->numel() != p.numel() || k->scalar_type() != p.scalar_type()) return std::nullopt;
-  return k;
-}
-
-at::Tensor grad_like(const at::Tensor& p, const at::Tensor& g) {
-  TORCH_CHECK(g.scalar_type() == p.scalar_type(), "optimi_amd: gradient dtype ", g.scalar_type(), " differs from parameter dtype ", p.scalar_type());
-  if (g.strides() == p.strides()) return g;
-  return at::empty_like(p).copy_(g);
-}
-
-uint32_t base_flags(bool kahan_sum, bool update) { return (kahan_sum ? OPTIMI_KAHAN : 0u) | (update ? OPTIMI_UPDATE : 0u); }
-
-void adam_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
-                  const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
-                  double weight_decay, double eps, bool decouple_wd, bool decouple_lr, std::optional<double> max_lr,
-                  bool kahan_sum, bool update) {
-  const int64_t t = tick(step);
-  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
-  if (weight_decay != 0) {
-    if (decouple_lr) weight_decay = 1 - (lr / max_lr.value()) * weight_decay;
-    else if (decouple_wd) weight_decay = 1 - lr * weight_decay;
-  }
-  const uint32_t flags = base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u);
-  adam_single(p, grad_like(p, g), m, v, real_kahan(p, k), lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps, flags);
-}
-
-void lion_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const std::optional<at::Tensor>& k,
-                  double lr, double beta1, double beta2, double weight_decay, bool decouple_lr,
-                  std::optional<double> max_lr, bool kahan_sum, bool update) {
-  if (weight_decay != 0) weight_decay = decouple_lr ? 1 - (lr / max_lr.value()) * weight_decay : 1 - lr * weight_decay;
-  lion_single(p, grad_like(p, g), m, real_kahan(p, k), lr, 1 - beta1, 1 - beta2, weight_decay, base_flags(kahan_sum, update));
-}
-
-void stableadamw_release(Group& group, const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
-                         const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
-                         double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum,
-                         bool update) {
-  const int64_t t = tick(step);
-  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
-  const uint32_t flags = base_flags(kahan_sum, update) | (decouple_lr ? OPTIMI_DECOUPLE_LR : 0u);
-  stableadamw_single(group, p, grad_like(p, g), m, v, real_kahan(p, k), lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps,
-                     (decouple_lr && max_lr.has_value()) ? *max_lr : 0.0, flags);
-}
-
-void adan_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& df, const at::Tensor& n,
-                  const at::Tensor& pg, const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1,
-                  double beta2, double beta3, double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr,
-                  bool adam_wd, bool kahan_sum, bool update) {
-  const int64_t t = tick(step);
-  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t), b3h = debias_beta(beta3, t);
-  if (weight_decay != 0) {
-    weight_decay = decouple_lr ? (lr / max_lr.value()) * weight_decay : lr * weight_decay;
-    weight_decay = adam_wd ? 1 - weight_decay : 1 + weight_decay;
-  }
-  const uint32_t flags = base_flags(kahan_sum, update) | (adam_wd ? OPTIMI_ADAM_WD : 0u);
-  adan_single(p, grad_like(p, g), m, df, n, pg, real_kahan(p, k), lr, 1 - b1h, beta2, 1 - b2h, b3h, 1 - b3h, eps, weight_decay,
-              flags);
-}
-
 void sgd_single(const at::Tensor& p, const at::Tensor& g, const std::optional<at::Tensor>& m,
                 const std::optional<at::Tensor>& kahan_comp, double lr, double momentum, double weight_decay, uint32_t flags) {
   One o = prepare_one(p, kahan_comp, flags);
@@ -446,6 +367,20 @@ void ranger_single(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m
                "optimi_hip_ranger_single");
 }
 
+// ---- gradient-release fast path --------------------------------------------------------
+// One call per parameter from the post-accumulate-grad hook: advances the parameter's int32
+// CPU step counter, forms the step scalars in double exactly as the functional forms do in
+// Python (optimi/adam.py:260-273, lion.py:226-235, stableadamw.py:326-332, adan.py:289-309)
+// and either launches the per-tensor kernel or, for a small tensor, parks the step in a
+// ReleaseQueue that launches many of them as one list.  std::pow(double, double) is libm's
+// pow, the function CPython's float ** int ends in, so the scalars are bit-identical to the
+// Python path.
+
+double debias_beta(double beta, int64_t step) {  // optimi/utils.py:31-36
+  const double bt = std::pow(beta, (double)step);
+  return (bt - beta) / (bt - 1.0);
+}
+
 // RAdam's variance rectification term; negative = not yet rectified (optimi/radam.py:269-277).
 double rectification(double beta2, int64_t step) {
   const double rho_inf = 2 / (1 - beta2) - 1;
@@ -455,22 +390,259 @@ double rectification(double beta2, int64_t step) {
   return -1.0;
 }
 
-void sgd_release(const at::Tensor& p, const at::Tensor& g, const std::optional<at::Tensor>& m,
-                 const std::optional<at::Tensor>& k, double lr, double momentum, double weight_decay, bool dampening,
-                 bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update) {
+int64_t tick(const at::Tensor& step) {
+  TORCH_CHECK(step.device().is_cpu() && step.scalar_type() == at::kInt && step.numel() == 1,
+              "optimi_amd: the step counter must be a one-element int32 CPU tensor");
+  int32_t* s = step.data_ptr<int32_t>();
+  *s += 1;
+  return *s;
+}
+
+// The Kahan buffer if it is one: placeholders (one element, maybe another dtype) and None count as absent.
+std::optional<at::Tensor> real_kahan(const at::Tensor& p, const std::optional<at::Tensor>& k) {
+  if (!k.has_value() || !k->defined() || k->numel() != p.numel() || k->scalar_type() != p.scalar_type()) return std::nullopt;
+  return k;
+}
+
+at::Tensor grad_like(const at::Tensor& p, const at::Tensor& g) {
+  TORCH_CHECK(g.scalar_type() == p.scalar_type(), "optimi_amd: gradient dtype ", g.scalar_type(), " differs from parameter dtype ", p.scalar_type());
+  if (g.strides() == p.strides()) return g;
+  return at::empty_like(p).copy_(g);
+}
+
+uint32_t base_flags(bool kahan_sum, bool update) { return (kahan_sum ? OPTIMI_KAHAN : 0u) | (update ? OPTIMI_UPDATE : 0u); }
+
+// One per-tensor step, ready to launch: the tensors in the order the ABI's entry point for
+// `kind` takes them (the parameter first, the Kahan buffer last; absent = nullopt) and the
+// scalars in the order it takes them.
+enum Kind { ADAM, LION, STABLEADAMW, ADAN, SGD, RADAM, RANGER };
+constexpr int kMaxTensors = 7, kMaxScalars = 8;
+constexpr int kTensorsOf[] = {5, 4, 5, 7, 4, 5, 6};
+constexpr int kScalarsOf[] = {6, 4, 7, 8, 3, 7, 8};
+
+struct StepCall {
+  Kind kind;
+  uint32_t flags = 0;
+  std::optional<at::Tensor> t[kMaxTensors];
+  double s[kMaxScalars] = {0, 0, 0, 0, 0, 0, 0, 0};
+  const at::Tensor& param() const { return *t[0]; }
+  const std::optional<at::Tensor>& kahan() const { return t[kTensorsOf[kind] - 1]; }
+};
+
+void launch_now(const StepCall& c, Group* stable_group) {
+  const auto& t = c.t;
+  const double* s = c.s;
+  switch (c.kind) {
+    case ADAM: adam_single(*t[0], *t[1], *t[2], *t[3], t[4], s[0], s[1], s[2], s[3], s[4], s[5], c.flags); break;
+    case LION: lion_single(*t[0], *t[1], *t[2], t[3], s[0], s[1], s[2], s[3], c.flags); break;
+    case STABLEADAMW:
+      TORCH_CHECK(stable_group, "optimi_amd: StableAdamW needs a launch workspace");
+      stableadamw_single(*stable_group, *t[0], *t[1], *t[2], *t[3], t[4], s[0], s[1], s[2], s[3], s[4], s[5], s[6], c.flags);
+      break;
+    case ADAN: adan_single(*t[0], *t[1], *t[2], *t[3], *t[4], *t[5], t[6], s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], c.flags); break;
+    case SGD: sgd_single(*t[0], *t[1], t[2], t[3], s[0], s[1], s[2], c.flags); break;
+    case RADAM: radam_single(*t[0], *t[1], *t[2], *t[3], t[4], s[0], s[1], s[2], s[3], s[4], s[5], s[6], c.flags); break;
+    case RANGER: ranger_single(*t[0], *t[1], *t[2], *t[3], *t[4], t[5], s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], c.flags); break;
+  }
+}
+
+// Parks the steps of small tensors and launches them together, as one list per run of steps
+// that share everything but their tensors (optimizer, dtype, device, stream, flags and every
+// scalar - which includes the step count through the debiased betas).  A tensor of a few
+// thousand elements costs far more to launch than to update, so a model with thousands of
+// them is bound by launches; one list launch replaces up to `max_tensors` of them.  The queue
+// keeps each parked gradient alive until its launch; `max_total` bounds how many elements
+// that may be.  Results are those of the per-tensor launches, bit for bit.
+class ReleaseQueue {
+ public:
+  ReleaseQueue(int64_t max_numel, int64_t max_tensors, int64_t max_total)
+      : max_numel_(max_numel), max_tensors_(max_tensors), max_total_(max_total) {}
+  ~ReleaseQueue() {
+    // steps still parked are dropped, never launched from a destructor (the device may be gone)
+  }
+
+  bool wants(const StepCall& c) const { return c.param().numel() <= max_numel_; }
+  int64_t pending() const { return (int64_t)batch_.size(); }
+
+  void add(StepCall&& c) {
+    validate(c);
+    const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(c.param().device().index()).stream();
+    if (!batch_.empty() && (!same_run(c, stream) || seen_.count(c.param().data_ptr()))) flush();
+    if (batch_.empty()) stream_ = stream;
+    total_ += c.param().numel();
+    seen_.insert(c.param().data_ptr());
+    batch_.push_back(std::move(c));
+    if ((int64_t)batch_.size() >= max_tensors_ || total_ >= max_total_) flush();
+  }
+
+  void flush() {
+    if (batch_.empty()) return;
+    std::vector<StepCall> batch;
+    batch.swap(batch_);  // the queue is empty again whatever happens below
+    seen_.clear();
+    total_ = 0;
+    const StepCall& c0 = batch[0];
+    const int n = (int)batch.size(), nt = kTensorsOf[c0.kind];
+    const int dtype = dtype_code(c0.param());
+    const bool kahan = c0.kahan().has_value();
+    std::vector<void*> ptr[kMaxTensors];
+    std::vector<int64_t> numel((size_t)n);
+    for (int a = 0; a < nt; ++a) ptr[a].resize((size_t)n, nullptr);
+    for (int i = 0; i < n; ++i) {
+      numel[(size_t)i] = batch[(size_t)i].param().numel();
+      for (int a = 0; a < nt; ++a)
+        if (batch[(size_t)i].t[a].has_value()) ptr[a][(size_t)i] = batch[(size_t)i].t[a]->data_ptr();
+    }
+    auto arr = [&](int a) { return (void* const*)ptr[a].data(); };
+    auto carr = [&](int a) { return (const void* const*)ptr[a].data(); };
+    auto opt = [&](int a, bool present) { return present ? (void* const*)ptr[a].data() : nullptr; };
+    const double* s = c0.s;
+    optimi_group* g = group_.get();
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(c0.param().device());
+    int rc = 0;
+    const char* what = "";
+    switch (c0.kind) {
+      case ADAM:
+        rc = optimi_hip_adam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], c0.flags, stream_);
+        what = "optimi_hip_adam_multi";
+        break;
+      case LION:
+        rc = optimi_hip_lion_multi(g, n, arr(0), carr(1), arr(2), opt(3, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], c0.flags, stream_);
+        what = "optimi_hip_lion_multi";
+        break;
+      case STABLEADAMW:
+        rc = optimi_hip_stableadamw_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], c0.flags, stream_);
+        what = "optimi_hip_stableadamw_multi";
+        break;
+      case ADAN:
+        rc = optimi_hip_adan_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), arr(5), opt(6, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], c0.flags, stream_);
+        what = "optimi_hip_adan_multi";
+        break;
+      case SGD:
+        rc = optimi_hip_sgd_multi(g, n, arr(0), carr(1), opt(2, c0.t[2].has_value()), opt(3, kahan), numel.data(), dtype, s[0], s[1], s[2], c0.flags, stream_);
+        what = "optimi_hip_sgd_multi";
+        break;
+      case RADAM:
+        rc = optimi_hip_radam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], c0.flags, stream_);
+        what = "optimi_hip_radam_multi";
+        break;
+      case RANGER:
+        rc = optimi_hip_ranger_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), opt(5, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], c0.flags, stream_);
+        what = "optimi_hip_ranger_multi";
+        break;
+    }
+    check_status(rc, what);
+  }
+
+ private:
+  // what the per-tensor entry points check before they launch
+  static void validate(const StepCall& c) {
+    static const char* const names[] = {"param", "grad", "state", "state", "state", "state", "state"};
+    const at::Tensor& p = c.param();
+    check_param(p);
+    (void)dtype_code(p);
+    for (int a = 1; a < kTensorsOf[c.kind]; ++a)
+      if (c.t[a].has_value()) check_like(p, *c.t[a], names[a]);
+  }
+
+  bool same_run(const StepCall& c, hipStream_t stream) const {
+    const StepCall& c0 = batch_[0];
+    if (c.kind != c0.kind || c.flags != c0.flags || stream != stream_) return false;
+    if (c.param().scalar_type() != c0.param().scalar_type() || c.param().device() != c0.param().device()) return false;
+    if (std::memcmp(c.s, c0.s, sizeof(c.s)) != 0) return false;
+    for (int a = 0; a < kTensorsOf[c.kind]; ++a)
+      if (c.t[a].has_value() != c0.t[a].has_value()) return false;
+    return true;
+  }
+
+  int64_t max_numel_, max_tensors_, max_total_;
+  Group group_;
+  std::vector<StepCall> batch_;
+  std::unordered_set<void*> seen_;
+  int64_t total_ = 0;
+  hipStream_t stream_ = nullptr;
+};
+
+// Parks the step when there is a queue and the tensor is small enough for it, otherwise
+// launches it.  Returns whether the step was parked (the caller then owes the queue a flush).
+bool submit(StepCall&& c, ReleaseQueue* queue, Group* stable_group = nullptr) {
+  if (queue && queue->wants(c)) {
+    queue->add(std::move(c));
+    return queue->pending() > 0;
+  }
+  launch_now(c, stable_group);
+  return false;
+}
+
+bool adam_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
+                  const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
+                  double weight_decay, double eps, bool decouple_wd, bool decouple_lr, std::optional<double> max_lr,
+                  bool kahan_sum, bool update, ReleaseQueue* queue) {
+  const int64_t t = tick(step);
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
   if (weight_decay != 0) {
     if (decouple_lr) weight_decay = 1 - (lr / max_lr.value()) * weight_decay;
     else if (decouple_wd) weight_decay = 1 - lr * weight_decay;
   }
-  const uint32_t flags = base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u) |
-                         (dampening ? OPTIMI_DAMPENING : 0u);
-  sgd_single(p, grad_like(p, g), momentum != 0 ? real_kahan(p, m) : std::nullopt, real_kahan(p, k), lr, momentum, weight_decay, flags);
+  StepCall c{ADAM, base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u),
+             {p, grad_like(p, g), m, v, real_kahan(p, k)}, {lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps}};
+  return submit(std::move(c), queue);
 }
 
-void ranger_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
+bool lion_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const std::optional<at::Tensor>& k,
+                  double lr, double beta1, double beta2, double weight_decay, bool decouple_lr,
+                  std::optional<double> max_lr, bool kahan_sum, bool update, ReleaseQueue* queue) {
+  if (weight_decay != 0) weight_decay = decouple_lr ? 1 - (lr / max_lr.value()) * weight_decay : 1 - lr * weight_decay;
+  StepCall c{LION, base_flags(kahan_sum, update), {p, grad_like(p, g), m, real_kahan(p, k)}, {lr, 1 - beta1, 1 - beta2, weight_decay}};
+  return submit(std::move(c), queue);
+}
+
+bool stableadamw_release(Group& group, const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
+                         const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
+                         double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum,
+                         bool update, ReleaseQueue* queue) {
+  const int64_t t = tick(step);
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
+  StepCall c{STABLEADAMW, base_flags(kahan_sum, update) | (decouple_lr ? OPTIMI_DECOUPLE_LR : 0u),
+             {p, grad_like(p, g), m, v, real_kahan(p, k)},
+             {lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps, (decouple_lr && max_lr.has_value()) ? *max_lr : 0.0}};
+  return submit(std::move(c), queue, &group);
+}
+
+bool adan_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& df, const at::Tensor& n,
+                  const at::Tensor& pg, const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1,
+                  double beta2, double beta3, double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr,
+                  bool adam_wd, bool kahan_sum, bool update, ReleaseQueue* queue) {
+  const int64_t t = tick(step);
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t), b3h = debias_beta(beta3, t);
+  if (weight_decay != 0) {
+    weight_decay = decouple_lr ? (lr / max_lr.value()) * weight_decay : lr * weight_decay;
+    weight_decay = adam_wd ? 1 - weight_decay : 1 + weight_decay;
+  }
+  StepCall c{ADAN, base_flags(kahan_sum, update) | (adam_wd ? OPTIMI_ADAM_WD : 0u),
+             {p, grad_like(p, g), m, df, n, pg, real_kahan(p, k)},
+             {lr, 1 - b1h, beta2, 1 - b2h, b3h, 1 - b3h, eps, weight_decay}};
+  return submit(std::move(c), queue);
+}
+
+bool sgd_release(const at::Tensor& p, const at::Tensor& g, const std::optional<at::Tensor>& m,
+                 const std::optional<at::Tensor>& k, double lr, double momentum, double weight_decay, bool dampening,
+                 bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update,
+                 ReleaseQueue* queue) {
+  if (weight_decay != 0) {
+    if (decouple_lr) weight_decay = 1 - (lr / max_lr.value()) * weight_decay;
+    else if (decouple_wd) weight_decay = 1 - lr * weight_decay;
+  }
+  StepCall c{SGD, base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u) | (dampening ? OPTIMI_DAMPENING : 0u),
+             {p, grad_like(p, g), momentum != 0 ? real_kahan(p, m) : std::nullopt, real_kahan(p, k)}, {lr, momentum, weight_decay}};
+  return submit(std::move(c), queue);
+}
+
+bool ranger_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
                     const std::optional<at::Tensor>& la, const std::optional<at::Tensor>& k, const at::Tensor& step, double lr,
                     double beta1, double beta2, double weight_decay, double eps, int64_t sync_every, double alpha,
-                    bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update) {
+                    bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update,
+                    ReleaseQueue* queue) {
   // la = None makes this RAdam (optimi/radam.py:214-322); with la it is Ranger (optimi/ranger.py:230-344)
   const int64_t t = tick(step);
   const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
@@ -481,14 +653,14 @@ void ranger_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& 
   }
   uint32_t flags = base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u) |
                    (rect >= 0 ? OPTIMI_RECTIFY : 0u);
+  const double r = rect >= 0 ? rect : 0.0;
   if (la.has_value()) {
     if (t % sync_every == 0) flags |= OPTIMI_LOOKAHEAD;
-    ranger_single(p, grad_like(p, g), m, v, *la, real_kahan(p, k), lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps,
-                  rect >= 0 ? rect : 0.0, alpha, flags);
-  } else {
-    radam_single(p, grad_like(p, g), m, v, real_kahan(p, k), lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps,
-                 rect >= 0 ? rect : 0.0, flags);
+    StepCall c{RANGER, flags, {p, grad_like(p, g), m, v, *la, real_kahan(p, k)}, {lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps, r, alpha}};
+    return submit(std::move(c), queue);
   }
+  StepCall c{RADAM, flags, {p, grad_like(p, g), m, v, real_kahan(p, k)}, {lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps, r}};
+  return submit(std::move(c), queue);
 }
 
 }  // namespace
@@ -505,6 +677,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.attr("LOOKAHEAD") = (uint32_t)OPTIMI_LOOKAHEAD;
   mod.def("abi_version", &optimi_hip_version);
   py::class_<Group>(mod, "Group").def(py::init<>());
+  py::class_<ReleaseQueue>(mod, "ReleaseQueue")
+      .def(py::init<int64_t, int64_t, int64_t>(), py::arg("max_numel"), py::arg("max_tensors"), py::arg("max_total"))
+      .def("flush", &ReleaseQueue::flush)
+      .def("pending", &ReleaseQueue::pending);
   mod.def("adam_multi", &adam_multi);
   mod.def("lion_multi", &lion_multi);
   mod.def("stableadamw_multi", &stableadamw_multi);

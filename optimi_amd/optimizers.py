@@ -16,6 +16,7 @@ from warnings import warn
 
 import torch
 from torch import Tensor
+from torch.autograd import Variable
 from torch.optim.optimizer import Optimizer
 
 from torch.optim import optimizer as _torch_optimizer
@@ -51,6 +52,14 @@ class OptimiOptimizer(Optimizer):
     _setup_before_state = False             # StableAdamW resolves its backend before touching state
     _step_state_from_group = True           # per-parameter counter keyed on the group's gradient_release flag (Adan: on the call)
 
+    # Gradient release parks the steps of tensors with at most this many elements and launches
+    # them together when the backward pass ends (0 = launch every tensor on its own, from its
+    # hook).  Results are identical; a model with thousands of small tensors steps several times
+    # faster.  Set on the instance, or on the class, before the first backward pass.
+    gradient_release_coalesce = 65536
+    _QUEUE_MAX_TENSORS = 1024               # parked steps per launch
+    _QUEUE_MAX_ELEMENTS = 1 << 24           # parked gradient elements kept alive at most
+
     def __init__(self, params: Iterable[Tensor] | Iterable[dict], defaults: dict[str, Any]):
         if not 0.0 <= defaults["lr"]:
             raise ValueError(f"Invalid learning rate: lr={defaults['lr']}")
@@ -79,6 +88,8 @@ class OptimiOptimizer(Optimizer):
 
         self._optimizer_accumulation = False
         self._hip_groups: dict = {}
+        self._release_queue = None
+        self._flush_scheduled = False
 
         if self.defaults["gradient_release"]:
             self.defaults["foreach"] = False
@@ -92,12 +103,20 @@ class OptimiOptimizer(Optimizer):
         state = super().__getstate__()
         state = dict(state)
         state.pop("_hip_groups", None)
+        state.pop("_release_queue", None)
+        state.pop("_flush_scheduled", None)
         return state
 
     def __setstate__(self, state):
         super().__setstate__(state)
         self.__dict__.setdefault("_hip_groups", {})
+        self.__dict__.setdefault("_release_queue", None)
+        self.__dict__.setdefault("_flush_scheduled", False)
         self.__dict__.setdefault("_optimizer_accumulation", False)
+
+    def state_dict(self):
+        self._flush_release()  # a checkpoint must not miss steps that are still parked
+        return super().state_dict()
 
     @property
     def optimizer_accumulation(self) -> bool:
@@ -181,6 +200,7 @@ class OptimiOptimizer(Optimizer):
                 loss = closure()
 
         if param is None:
+            self._flush_release()
             for group in self.param_groups:
                 params = self._collect(group)
                 if params and not group["triton"]:
@@ -202,9 +222,10 @@ class OptimiOptimizer(Optimizer):
         return loss
 
     # -- gradient-release fast path --------------------------------------------------------
-    def _release_call(self, ext, group, state, param, grad, update):
+    def _release_call(self, ext, group, state, param, grad, update, queue):
         """One native call that advances the parameter's step counter, forms the step scalars and
-        launches the per-tensor kernel.  Subclasses forward their hyper-parameters."""
+        launches the per-tensor kernel, or parks the step in ``queue`` when the tensor is small
+        (then it returns True).  Subclasses forward their hyper-parameters."""
         raise NotImplementedError
 
     def _has_step_hooks(self) -> bool:
@@ -231,8 +252,25 @@ class OptimiOptimizer(Optimizer):
         if not group["triton"]:
             raise RuntimeError("optimi_amd: parameter is not eligible for the HIP backend and there is no other backend")
         backend.check_supported(param)
-        self._release_call(backend.ext(), group, state, param, param.grad, not self._optimizer_accumulation)
+        ext = backend.ext()
+        # steps are parked only inside a backward pass, whose end launches them
+        queue = None
+        if self.gradient_release_coalesce > 0 and torch._C._current_graph_task_id() != -1:
+            queue = self._release_queue
+            if queue is None:
+                queue = self._release_queue = ext.ReleaseQueue(self.gradient_release_coalesce, self._QUEUE_MAX_TENSORS,
+                                                               self._QUEUE_MAX_ELEMENTS)
+        parked = self._release_call(ext, group, state, param, param.grad, not self._optimizer_accumulation, queue)
         param.grad = None
+        if parked and not self._flush_scheduled:
+            Variable._execution_engine.queue_callback(self._flush_release)
+            self._flush_scheduled = True
+
+    def _flush_release(self):
+        """Launches the gradient-release steps that are still parked."""
+        self._flush_scheduled = False
+        if self._release_queue is not None:
+            self._release_queue.flush()
 
     @torch._disable_dynamo
     def zero_grad(self, set_to_none: bool = True, param: Tensor | None = None):
@@ -243,6 +281,7 @@ class OptimiOptimizer(Optimizer):
             param: Resets the gradients of the passed `param`. For use with `gradient_release=True`.
         """
         if param is None:
+            self._flush_release()
             super().zero_grad(set_to_none=set_to_none)
         elif param.grad is not None:
             if set_to_none:
@@ -315,10 +354,10 @@ class Adam(OptimiOptimizer):
                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
 
-    def _release_call(self, ext, group, state, param, grad, update):
-        ext.adam_release(param, grad, state["exp_avg"], state["exp_avg_sq"], state["kahan_comp"], state["step"], group["lr"],
+    def _release_call(self, ext, group, state, param, grad, update, queue):
+        return ext.adam_release(param, grad, state["exp_avg"], state["exp_avg_sq"], state["kahan_comp"], state["step"], group["lr"],
                          group["beta1"], group["beta2"], group["weight_decay"], group["eps"], group["decouple_wd"],
-                         group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update)
+                         group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update, queue)
 
 
 class AdamW(Adam):
@@ -391,9 +430,9 @@ class Lion(OptimiOptimizer):
                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
 
-    def _release_call(self, ext, group, state, param, grad, update):
-        ext.lion_release(param, grad, state["exp_avg"], state["kahan_comp"], group["lr"], group["beta1"], group["beta2"],
-                         group["weight_decay"], group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update)
+    def _release_call(self, ext, group, state, param, grad, update, queue):
+        return ext.lion_release(param, grad, state["exp_avg"], state["kahan_comp"], group["lr"], group["beta1"], group["beta2"],
+                         group["weight_decay"], group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update, queue)
 
 
 def _restore_scratch_state(optim: OptimiOptimizer):
@@ -464,11 +503,11 @@ class StableAdamW(OptimiOptimizer):
                       _groups=self._hip_groups)
 
 
-    def _release_call(self, ext, group, state, param, grad, update):
+    def _release_call(self, ext, group, state, param, grad, update, queue):
         grp = F._workspace(self._hip_groups, param.device, param.dtype, "stableadamw_single")
-        ext.stableadamw_release(grp, param, grad, state["exp_avg"], state["exp_avg_sq"], state["kahan_comp"], state["step"],
+        return ext.stableadamw_release(grp, param, grad, state["exp_avg"], state["exp_avg_sq"], state["kahan_comp"], state["step"],
                                 group["lr"], group["beta1"], group["beta2"], group["weight_decay"], group["eps"],
-                                group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update)
+                                group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update, queue)
 
 
 class Adan(OptimiOptimizer):
@@ -533,12 +572,12 @@ class Adan(OptimiOptimizer):
                foreach=False, triton=True, gradient_release=gradient_release,
                optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
-    def _release_call(self, ext, group, state, param, grad, update):
+    def _release_call(self, ext, group, state, param, grad, update, queue):
         # adam_wd is not forwarded, as in step() above
-        ext.adan_release(param, grad, state["exp_avg"], state["exp_avg_diff"], state["exp_avg_sq"], state["prev_grad"],
+        return ext.adan_release(param, grad, state["exp_avg"], state["exp_avg_diff"], state["exp_avg_sq"], state["prev_grad"],
                          state["kahan_comp"], state["step"], group["lr"], group["beta1"], group["beta2"], group["beta3"],
                          group["weight_decay"], group["eps"], group["decouple_lr"], group["max_lr"], False,
-                         bool(group["kahan_sum"]), update)
+                         bool(group["kahan_sum"]), update, queue)
 
 
 class SGD(OptimiOptimizer):
@@ -613,10 +652,10 @@ class SGD(OptimiOptimizer):
               kahan_sum=group["kahan_sum"], foreach=False, triton=True, gradient_release=gradient_release,
               optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
-    def _release_call(self, ext, group, state, param, grad, update):
-        ext.sgd_release(param, grad, state["exp_avg"], state["kahan_comp"], group["lr"], group["momentum"],
+    def _release_call(self, ext, group, state, param, grad, update, queue):
+        return ext.sgd_release(param, grad, state["exp_avg"], state["kahan_comp"], group["lr"], group["momentum"],
                         group["weight_decay"], group["dampening"], group["decouple_wd"], group["decouple_lr"],
-                        group["max_lr"], bool(group["kahan_sum"]), update)
+                        group["max_lr"], bool(group["kahan_sum"]), update, queue)
 
 
 class RAdam(OptimiOptimizer):
@@ -665,10 +704,10 @@ class RAdam(OptimiOptimizer):
                 max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
                 gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
-    def _release_call(self, ext, group, state, param, grad, update):
-        ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], None, state["kahan_comp"], state["step"],
+    def _release_call(self, ext, group, state, param, grad, update, queue):
+        return ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], None, state["kahan_comp"], state["step"],
                            group["lr"], group["beta1"], group["beta2"], group["weight_decay"], group["eps"], 1, 0.0,
-                           group["decouple_wd"], group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update)
+                           group["decouple_wd"], group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update, queue)
 
 
 class Ranger(OptimiOptimizer):
@@ -725,8 +764,8 @@ class Ranger(OptimiOptimizer):
                  kahan_sum=group["kahan_sum"], foreach=False, triton=True, gradient_release=gradient_release,
                  optimizer_accumulation=accumulate, _groups=self._hip_groups)
 
-    def _release_call(self, ext, group, state, param, grad, update):
-        ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], state["la_param"], state["kahan_comp"],
+    def _release_call(self, ext, group, state, param, grad, update, queue):
+        return ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], state["la_param"], state["kahan_comp"],
                            state["step"], group["lr"], group["beta1"], group["beta2"], group["weight_decay"],
                            group["eps"], group["k"], group["alpha"], group["decouple_wd"], group["decouple_lr"],
-                           group["max_lr"], bool(group["kahan_sum"]), update)
+                           group["max_lr"], bool(group["kahan_sum"]), update, queue)

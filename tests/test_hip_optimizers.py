@@ -224,3 +224,67 @@ def test_step_hooks_still_fire_under_gradient_release(hip_device):
     loss_step(model, torch.bfloat16, hip_device, torch.Generator().manual_seed(1))
     assert len(calls) == len(params)
     optimi_amd.remove_gradient_release(model)
+
+
+class ManySmall(torch.nn.Module):
+    """Parameters of many sizes, most below the coalescing limit, two above it, two of them fp32;
+    the loss gives every parameter a dense, non-trivial gradient."""
+
+    SIZES = [5, 64, 513, 4096, 70000, 8191, 1, 300, 65536, 65537, 1000, 17, 2048, 9, 129, 33000]
+
+    def __init__(self, device, seed=0):
+        super().__init__()
+        gen = torch.Generator().manual_seed(seed)
+        self.ps = torch.nn.ParameterList()
+        for i, n in enumerate(self.SIZES):
+            dt = torch.float32 if i in (3, 11) else torch.bfloat16
+            self.ps.append(torch.nn.Parameter((torch.randn(n, generator=gen) * 0.02).to(dt).to(device)))
+        self.ws = [(torch.randn(n, generator=gen) * 1e-3).to(device) for n in self.SIZES]
+
+    def forward(self, scale):
+        return sum((p.float() * w).sum() for p, w in zip(self.ps, self.ws)) * scale
+
+
+@pytest.mark.parametrize("max_tensors", [1024, 3], ids=["one_flush", "flush_every_3"])
+@pytest.mark.parametrize("case", ["adamw", "adamw_declr", "lion", "stableadamw", "adan", "sgd", "radam", "ranger"])
+def test_coalesced_release_equals_per_tensor_launches(case, max_tensors, hip_device):
+    """Gradient release with small tensors parked and launched as lists (the default) gives the
+    bits of one launch per tensor from each hook, across accumulate-only and full steps, two
+    dtypes and tensors on both sides of the size limit."""
+    cls, _, hyper = CASES[case]
+    a, b = ManySmall(hip_device), ManySmall(hip_device)
+    parked, direct = cls(a.parameters(), gradient_release=True, **hyper), cls(b.parameters(), gradient_release=True, **hyper)
+    parked._QUEUE_MAX_TENSORS = max_tensors
+    direct.gradient_release_coalesce = 0
+    optimi_amd.prepare_for_gradient_release(a, parked)
+    optimi_amd.prepare_for_gradient_release(b, direct)
+    for it in range(8):
+        parked.optimizer_accumulation = direct.optimizer_accumulation = (it + 1) % 4 != 0
+        for model in (a, b):
+            model(1.0 + it).backward()
+        assert parked._release_queue.pending() == 0 and direct._release_queue is None
+        assert all(p.grad is None for p in a.parameters())
+    for i, (pa, pb) in enumerate(zip(a.parameters(), b.parameters())):
+        G.assert_bits_equal(pa, pb, f"{case} param {i}")
+        assert list(parked.state[pa].keys()) == list(direct.state[pb].keys())
+        for key, val in parked.state[pa].items():
+            if torch.is_tensor(val) and val.is_cuda and val.is_floating_point():
+                G.assert_bits_equal(val, direct.state[pb][key], f"{case} {key} {i}")
+        if "step" in parked.state[pa]:
+            assert int(parked.state[pa]["step"]) == int(direct.state[pb]["step"]) == 8
+    assert not torch.equal(next(a.parameters()), ManySmall(hip_device).ps[0]), "nothing was stepped"
+    optimi_amd.remove_gradient_release(a)
+    optimi_amd.remove_gradient_release(b)
+
+
+def test_release_outside_a_backward_pass_launches_at_once(hip_device):
+    """Steps are parked only inside a backward pass (its end launches them); a hook body called
+    by hand launches its tensor directly."""
+    p = torch.nn.Parameter((torch.randn(1000) * 0.02).bfloat16().to(hip_device))
+    before = p.detach().clone()
+    opt = optimi_amd.AdamW([p], lr=1e-3, gradient_release=True)
+    p.grad = torch.full_like(p, 1e-3)
+    opt._release(p)
+    assert opt._release_queue is None and p.grad is None
+    assert not torch.equal(p.detach(), before)
+    assert int(opt.state_dict()["state"][0]["step"]) == 1

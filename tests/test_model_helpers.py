@@ -57,7 +57,7 @@ class TinyLM(nn.Module):
         self.register_buffer("global_scale", torch.ones(1))
 
     def forward(self, x):
-        return self.head(self.norm(self.attn(self.tok_embeddings(x))))
+        return self.head(self.norm(self.attn(self.tok_embeddings(x).to(self.head.weight.dtype))))
 
 
 @pytest.mark.parametrize("cls", CLASSES)
