@@ -9,11 +9,18 @@
 
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/csrc/autograd/engine.h>
+#include <torch/csrc/autograd/graph_task.h>
+#include <torch/csrc/autograd/python_variable.h>
 #include <torch/extension.h>
 
 #include <cmath>
 #include <cstring>
+#include <memory>
+#include <mutex>
 #include <optional>
+#include <string>
+#include <unordered_map>
 #include <unordered_set>
 #include <vector>
 
@@ -453,7 +460,12 @@ void launch_now(const StepCall& c, Group* stable_group) {
 // them is bound by launches; one list launch replaces up to `max_tensors` of them.  The queue
 // keeps each parked gradient alive until its launch; `max_total` bounds how many elements
 // that may be.  Results are those of the per-tensor launches, bit for bit.
-class ReleaseQueue {
+//
+// Steps are parked only while a backward pass runs: the first one parked in a pass registers
+// a final callback with the autograd engine, which launches whatever is parked when the pass
+// has finished.  That callback may run on another thread than the hooks and without the GIL;
+// it touches tensors only.
+class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
  public:
   ReleaseQueue(int64_t max_numel, int64_t max_tensors, int64_t max_total)
       : max_numel_(max_numel), max_tensors_(max_tensors), max_total_(max_total) {}
@@ -461,10 +473,34 @@ class ReleaseQueue {
     // steps still parked are dropped, never launched from a destructor (the device may be gone)
   }
 
-  bool wants(const StepCall& c) const { return c.param().numel() <= max_numel_; }
-  int64_t pending() const { return (int64_t)batch_.size(); }
+  bool wants(const StepCall& c) const {
+    return c.param().numel() <= max_numel_ && torch::autograd::get_current_graph_task_id() != -1;
+  }
+  int64_t pending() {
+    std::lock_guard<std::recursive_mutex> lock(mutex_);
+    return (int64_t)batch_.size();
+  }
+
+  // Makes sure the running backward pass ends with a flush.
+  void schedule() {
+    std::lock_guard<std::recursive_mutex> lock(mutex_);
+    const int task = torch::autograd::get_current_graph_task_id();
+    if (task == -1 || task == scheduled_task_) return;
+    std::weak_ptr<ReleaseQueue> weak = weak_from_this();
+    torch::autograd::Engine::get_default_engine().queue_callback([weak] {
+      if (std::shared_ptr<ReleaseQueue> q = weak.lock()) {
+        {
+          std::lock_guard<std::recursive_mutex> inner(q->mutex_);
+          q->scheduled_task_ = -1;
+        }
+        q->flush();
+      }
+    });
+    scheduled_task_ = task;
+  }
 
   void add(StepCall&& c) {
+    std::lock_guard<std::recursive_mutex> lock(mutex_);
     validate(c);
     const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(c.param().device().index()).stream();
     if (!batch_.empty() && (!same_run(c, stream) || seen_.count(c.param().data_ptr()))) flush();
@@ -476,6 +512,7 @@ class ReleaseQueue {
   }
 
   void flush() {
+    std::lock_guard<std::recursive_mutex> lock(mutex_);
     if (batch_.empty()) return;
     std::vector<StepCall> batch;
     batch.swap(batch_);  // the queue is empty again whatever happens below
@@ -497,8 +534,10 @@ class ReleaseQueue {
     auto carr = [&](int a) { return (const void* const*)ptr[a].data(); };
     auto opt = [&](int a, bool present) { return present ? (void* const*)ptr[a].data() : nullptr; };
     const double* s = c0.s;
-    optimi_group* g = group_.get();
     c10::hip::HIPGuardMasqueradingAsCUDA guard(c0.param().device());
+    std::unique_ptr<Group>& slot = groups_[c0.param().device().index()];  // a workspace lives on one device
+    if (!slot) slot = std::make_unique<Group>();  // made on first use: a queue may exist before any device work
+    optimi_group* g = slot->get();
     int rc = 0;
     const char* what = "";
     switch (c0.kind) {
@@ -556,19 +595,22 @@ class ReleaseQueue {
   }
 
   int64_t max_numel_, max_tensors_, max_total_;
-  Group group_;
+  std::recursive_mutex mutex_;
+  int scheduled_task_ = -1;  // the backward pass that already carries the flush callback
+  std::unordered_map<int, std::unique_ptr<Group>> groups_;
   std::vector<StepCall> batch_;
   std::unordered_set<void*> seen_;
   int64_t total_ = 0;
   hipStream_t stream_ = nullptr;
 };
 
-// Parks the step when there is a queue and the tensor is small enough for it, otherwise
-// launches it.  Returns whether the step was parked (the caller then owes the queue a flush).
+// Parks the step when there is a queue, a backward pass is running and the tensor is small
+// enough, otherwise launches it.  Returns whether the step was parked.
 bool submit(StepCall&& c, ReleaseQueue* queue, Group* stable_group = nullptr) {
   if (queue && queue->wants(c)) {
     queue->add(std::move(c));
-    return queue->pending() > 0;
+    queue->schedule();
+    return true;
   }
   launch_now(c, stable_group);
   return false;
@@ -663,6 +705,250 @@ bool ranger_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& 
   return submit(std::move(c), queue);
 }
 
+
+// ---- the post-accumulate-grad hook itself ------------------------------------------------
+// What optimi's hook does in Python for every parameter of every backward pass - look the
+// parameter's state and group up, read the hyper-parameters, step, free the gradient
+// (optimi/gradientrelease.py:13-15, adam.py:183-208, optimizer.py:96-114) - done here without a
+// Python frame.  Hyper-parameters are read from the group dict on every call, so schedulers
+// that rewrite them are seen.  State tensors are cached per parameter and re-validated by
+// identity against the state dict on every call; a parameter seen for the first time, or whose
+// state changed, goes through the optimizer's Python method `_release_entry`, which creates
+// the state exactly as step(param=...) would.  When step hooks are registered on the optimizer
+// the Python path runs instead, so they fire.
+class ReleaseHookCore {
+ public:
+  ReleaseHookCore(const py::object& optimizer, int kind, std::shared_ptr<ReleaseQueue> queue)
+      : optimizer_(py::weakref(optimizer)), kind_((Kind)kind), queue_(std::move(queue)) {
+    TORCH_CHECK(kind >= ADAM && kind <= RANGER, "optimi_amd: unknown optimizer kind ", kind);
+    static const char* const keys[][5] = {
+        {"exp_avg", "exp_avg_sq", "kahan_comp", nullptr, nullptr},               // ADAM
+        {"exp_avg", "kahan_comp", nullptr, nullptr, nullptr},                    // LION
+        {"exp_avg", "exp_avg_sq", "kahan_comp", nullptr, nullptr},               // STABLEADAMW
+        {"exp_avg", "exp_avg_diff", "exp_avg_sq", "prev_grad", "kahan_comp"},    // ADAN
+        {"exp_avg", "kahan_comp", nullptr, nullptr, nullptr},                    // SGD
+        {"exp_avg", "exp_avg_sq", "kahan_comp", nullptr, nullptr},               // RADAM
+        {"exp_avg", "exp_avg_sq", "la_param", "kahan_comp", nullptr},            // RANGER
+    };
+    for (int i = 0; i < 5 && keys[kind][i]; ++i) state_keys_.emplace_back(keys[kind][i]);
+    has_step_ = kind_ != LION && kind_ != SGD;
+    rebind();
+  }
+
+  // Forgets every cached parameter and re-reads the optimizer's hook tables; the optimizer
+  // calls this whenever its state or groups are replaced wholesale (load_state_dict).
+  void invalidate() {
+    entries_.clear();
+    rebind();
+  }
+
+  void call(const py::handle& param_h) {
+    TORCH_CHECK(THPVariable_Check(param_h.ptr()), "optimi_amd: the gradient release hook takes the parameter");
+    py::object optimizer = optimizer_();
+    TORCH_CHECK(!optimizer.is_none(), "optimi_amd: the optimizer of this gradient release hook no longer exists");
+    if (any_step_hooks()) {
+      optimizer.attr(k_.release)(param_h);
+      return;
+    }
+    const at::Tensor& p = THPVariable_Unpack(param_h.ptr());
+    Entry* e = find(p);
+    if (!e || !valid(*e)) e = refresh(optimizer, param_h, p);
+    const at::Tensor g = p.grad();
+    TORCH_CHECK(g.defined(), "optimi_amd: the gradient release hook ran on a parameter without a gradient");
+    at::NoGradGuard no_grad;
+    const bool update = !truthy(py::reinterpret_steal<py::object>(attr(optimizer.ptr(), k_.accumulation)).ptr());
+    PyObject* grp = e->group.ptr();
+    ReleaseQueue* q = queue_.get();
+    const auto& t = e->t;
+    switch (kind_) {
+      case ADAM:
+        adam_release(p, g, *t[0], *t[1], t[2], e->step, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2),
+                     num(grp, k_.weight_decay), num(grp, k_.eps), flag(grp, k_.decouple_wd), flag(grp, k_.decouple_lr),
+                     opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update, q);
+        break;
+      case LION:
+        lion_release(p, g, *t[0], t[1], num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2), num(grp, k_.weight_decay),
+                     flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update, q);
+        break;
+      case STABLEADAMW:
+        stableadamw_release(*e->workspace, p, g, *t[0], *t[1], t[2], e->step, num(grp, k_.lr), num(grp, k_.beta1),
+                            num(grp, k_.beta2), num(grp, k_.weight_decay), num(grp, k_.eps), flag(grp, k_.decouple_lr),
+                            opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update, q);
+        break;
+      case ADAN:  // adam_wd is not forwarded by the reference's class either (optimi/adan.py:186-208)
+        adan_release(p, g, *t[0], *t[1], *t[2], *t[3], t[4], e->step, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2),
+                     num(grp, k_.beta3), num(grp, k_.weight_decay), num(grp, k_.eps), flag(grp, k_.decouple_lr),
+                     opt_num(grp, k_.max_lr), false, flag(grp, k_.kahan_sum), update, q);
+        break;
+      case SGD:
+        sgd_release(p, g, t[0], t[1], num(grp, k_.lr), num(grp, k_.momentum), num(grp, k_.weight_decay),
+                    flag(grp, k_.dampening), flag(grp, k_.decouple_wd), flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr),
+                    flag(grp, k_.kahan_sum), update, q);
+        break;
+      case RADAM:
+        ranger_release(p, g, *t[0], *t[1], std::nullopt, t[2], e->step, num(grp, k_.lr), num(grp, k_.beta1),
+                       num(grp, k_.beta2), num(grp, k_.weight_decay), num(grp, k_.eps), 1, 0.0, flag(grp, k_.decouple_wd),
+                       flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update, q);
+        break;
+      case RANGER:
+        ranger_release(p, g, *t[0], *t[1], t[2], t[3], e->step, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2),
+                       num(grp, k_.weight_decay), num(grp, k_.eps), (int64_t)num(grp, k_.k), num(grp, k_.alpha),
+                       flag(grp, k_.decouple_wd), flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr),
+                       flag(grp, k_.kahan_sum), update, q);
+        break;
+    }
+    p.mutable_grad().reset();  // param.grad = None
+  }
+
+ private:
+  struct Entry {
+    c10::weak_intrusive_ptr<c10::TensorImpl> param;  // weak: a hook must not keep its parameter alive
+    py::object state, group, workspace_obj;
+    Group* workspace = nullptr;
+    PyObject* ids[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    PyObject* step_id = nullptr;
+    std::optional<at::Tensor> t[5];
+    at::Tensor step;
+    explicit Entry(const at::Tensor& p) : param(p.getIntrusivePtr()) {}
+  };
+
+  struct Names {
+    py::str release{"_release"}, entry{"_release_entry"}, accumulation{"_optimizer_accumulation"}, group{"group"}, step{"step"};
+    py::str lr{"lr"}, beta1{"beta1"}, beta2{"beta2"}, beta3{"beta3"}, weight_decay{"weight_decay"}, eps{"eps"};
+    py::str decouple_wd{"decouple_wd"}, decouple_lr{"decouple_lr"}, max_lr{"max_lr"}, kahan_sum{"kahan_sum"};
+    py::str momentum{"momentum"}, dampening{"dampening"}, k{"k"}, alpha{"alpha"};
+  };
+
+  static PyObject* attr(PyObject* obj, const py::str& name) {
+    PyObject* v = PyObject_GetAttr(obj, name.ptr());
+    if (!v) throw py::error_already_set();
+    return v;  // new reference
+  }
+  static PyObject* item(PyObject* dict, const py::str& key) {
+    PyObject* v = PyDict_GetItemWithError(dict, key.ptr());  // borrowed
+    if (!v) {
+      if (PyErr_Occurred()) throw py::error_already_set();
+      TORCH_CHECK(false, "optimi_amd: '", std::string(key), "' is missing from the parameter group");
+    }
+    return v;
+  }
+  static double as_double(PyObject* v) {
+    const double d = PyFloat_AsDouble(v);
+    if (d == -1.0 && PyErr_Occurred()) throw py::error_already_set();
+    return d;
+  }
+  static bool truthy(PyObject* v) {
+    const int r = PyObject_IsTrue(v);
+    if (r < 0) throw py::error_already_set();
+    return r == 1;
+  }
+  static double num(PyObject* dict, const py::str& key) { return as_double(item(dict, key)); }
+  static bool flag(PyObject* dict, const py::str& key) { return truthy(item(dict, key)); }
+  static std::optional<double> opt_num(PyObject* dict, const py::str& key) {
+    PyObject* v = item(dict, key);
+    if (v == Py_None) return std::nullopt;
+    return as_double(v);
+  }
+
+  void rebind() {
+    hook_tables_.clear();
+    py::object optimizer = optimizer_();
+    if (optimizer.is_none()) return;
+    py::module_ mod = py::module_::import("torch.optim.optimizer");
+    hook_tables_.push_back(optimizer.attr("_optimizer_step_pre_hooks"));
+    hook_tables_.push_back(optimizer.attr("_optimizer_step_post_hooks"));
+    hook_tables_.push_back(mod.attr("_global_optimizer_pre_hooks"));
+    hook_tables_.push_back(mod.attr("_global_optimizer_post_hooks"));
+  }
+
+  bool any_step_hooks() const {
+    for (const py::object& table : hook_tables_) {
+      const Py_ssize_t n = PyObject_Length(table.ptr());
+      if (n < 0) throw py::error_already_set();
+      if (n > 0) return true;
+    }
+    return false;
+  }
+
+  Entry* find(const at::Tensor& p) {
+    auto it = entries_.find(p.unsafeGetTensorImpl());
+    if (it == entries_.end()) return nullptr;
+    if (it->second.param.expired()) {  // another tensor lives at that address now
+      entries_.erase(it);
+      return nullptr;
+    }
+    return &it->second;
+  }
+
+  // every cached tensor is still the object the state dict holds
+  bool valid(const Entry& e) const {
+    PyObject* st = e.state.ptr();
+    for (size_t i = 0; i < state_keys_.size(); ++i)
+      if (PyDict_GetItemWithError(st, state_keys_[i].ptr()) != e.ids[i]) return false;
+    if (PyDict_GetItemWithError(st, k_.group.ptr()) != e.group.ptr()) return false;
+    if (has_step_ && PyDict_GetItemWithError(st, k_.step.ptr()) != e.step_id) return false;
+    return true;
+  }
+
+  Entry* refresh(const py::object& optimizer, const py::handle& param_h, const at::Tensor& p) {
+    PyErr_Clear();
+    // (state dict, group dict, launch workspace or None), state created and the backend checked
+    py::tuple made = optimizer.attr(k_.entry)(param_h);
+    Entry e(p);
+    e.state = made[0];
+    e.group = made[1];
+    e.workspace_obj = made[2];
+    TORCH_CHECK(PyDict_Check(e.state.ptr()) && PyDict_Check(e.group.ptr()), "optimi_amd: state and group must be dicts");
+    if (!e.workspace_obj.is_none()) e.workspace = &e.workspace_obj.cast<Group&>();
+    TORCH_CHECK(kind_ != STABLEADAMW || e.workspace, "optimi_amd: StableAdamW needs a launch workspace");
+    for (size_t i = 0; i < state_keys_.size(); ++i) {
+      PyObject* v = PyDict_GetItemWithError(e.state.ptr(), state_keys_[i].ptr());
+      TORCH_CHECK(v, "optimi_amd: optimizer state has no '", std::string(state_keys_[i]), "'");
+      e.ids[i] = v;
+      if (v != Py_None) {
+        TORCH_CHECK(THPVariable_Check(v), "optimi_amd: state '", std::string(state_keys_[i]), "' is not a tensor");
+        e.t[i] = THPVariable_Unpack(v);
+      }
+    }
+    // all but the last key (the Kahan buffer) and SGD's momentum buffer must be tensors
+    for (size_t i = 0; i + 1 < state_keys_.size(); ++i)
+      TORCH_CHECK(e.t[i].has_value() || kind_ == SGD, "optimi_amd: state '", std::string(state_keys_[i]), "' is None");
+    if (has_step_) {
+      PyObject* v = PyDict_GetItemWithError(e.state.ptr(), k_.step.ptr());
+      TORCH_CHECK(v && THPVariable_Check(v), "optimi_amd: the per-parameter step counter is missing");
+      e.step_id = v;
+      e.step = THPVariable_Unpack(v);
+    }
+    auto placed = entries_.insert_or_assign(p.unsafeGetTensorImpl(), std::move(e));
+    return &placed.first->second;
+  }
+
+  py::weakref optimizer_;
+  Kind kind_;
+  std::shared_ptr<ReleaseQueue> queue_;
+  bool has_step_ = true;
+  Names k_;
+  std::vector<py::str> state_keys_;
+  std::vector<py::object> hook_tables_;
+  std::unordered_map<c10::TensorImpl*, Entry> entries_;
+};
+
+// What is registered on the parameters: a handle that does not own the hook, so that
+// parameter -> hook -> cached state -> group -> parameter is not a cycle the garbage
+// collector cannot see.  The optimizer owns the ReleaseHookCore.
+class ReleaseHook {
+ public:
+  explicit ReleaseHook(const std::shared_ptr<ReleaseHookCore>& core) : core_(core) {}
+  void call(const py::handle& param) {
+    std::shared_ptr<ReleaseHookCore> core = core_.lock();
+    TORCH_CHECK(core, "optimi_amd: the optimizer of this gradient release hook no longer exists");
+    core->call(param);
+  }
+
+ private:
+  std::weak_ptr<ReleaseHookCore> core_;
+};
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
@@ -677,7 +963,21 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.attr("LOOKAHEAD") = (uint32_t)OPTIMI_LOOKAHEAD;
   mod.def("abi_version", &optimi_hip_version);
   py::class_<Group>(mod, "Group").def(py::init<>());
-  py::class_<ReleaseQueue>(mod, "ReleaseQueue")
+  py::class_<ReleaseHookCore, std::shared_ptr<ReleaseHookCore>>(mod, "ReleaseHookCore")
+      .def(py::init<const py::object&, int, std::shared_ptr<ReleaseQueue>>(), py::arg("optimizer"), py::arg("kind"), py::arg("queue"))
+      .def("invalidate", &ReleaseHookCore::invalidate)
+      .def("__call__", &ReleaseHookCore::call);
+  py::class_<ReleaseHook>(mod, "ReleaseHook")
+      .def(py::init<const std::shared_ptr<ReleaseHookCore>&>())
+      .def("__call__", &ReleaseHook::call);
+  mod.attr("KIND_ADAM") = (int)ADAM;
+  mod.attr("KIND_LION") = (int)LION;
+  mod.attr("KIND_STABLEADAMW") = (int)STABLEADAMW;
+  mod.attr("KIND_ADAN") = (int)ADAN;
+  mod.attr("KIND_SGD") = (int)SGD;
+  mod.attr("KIND_RADAM") = (int)RADAM;
+  mod.attr("KIND_RANGER") = (int)RANGER;
+  py::class_<ReleaseQueue, std::shared_ptr<ReleaseQueue>>(mod, "ReleaseQueue")
       .def(py::init<int64_t, int64_t, int64_t>(), py::arg("max_numel"), py::arg("max_tensors"), py::arg("max_total"))
       .def("flush", &ReleaseQueue::flush)
       .def("pending", &ReleaseQueue::pending);

@@ -3,7 +3,6 @@ accumulated, then free the gradient (optimi/gradientrelease.py:13-61)."""
 
 from __future__ import annotations
 
-from functools import partial
 from warnings import warn
 
 from torch import Tensor
@@ -15,7 +14,10 @@ __all__ = ["prepare_for_gradient_release", "remove_gradient_release"]
 
 
 def _gradient_release_hook(param: Tensor, optimizer: OptimiOptimizer):
-    # step(param=param) then zero_grad(param=param), in one native call per parameter
+    """What every registered hook does: ``step(param=param)`` then ``zero_grad(param=param)``
+    (optimi/gradientrelease.py:13-15).  The hooks registered below are the native form of this
+    function (state and group lookup, scalar prologue, launch or parking, freeing the gradient,
+    without a Python frame per parameter); this Python form gives the same results."""
     optimizer._release(param)
 
 
@@ -35,6 +37,7 @@ def prepare_for_gradient_release(model: Module, optimizer: OptimiOptimizer, igno
     if not optimizer.defaults["gradient_release"]:
         raise ValueError("`optimizer` must be initialized with `gradient_release=True`")
 
+    hook = optimizer._native_hook()
     registered = []
     for p in model.parameters():
         if not p.requires_grad:
@@ -46,8 +49,10 @@ def prepare_for_gradient_release(model: Module, optimizer: OptimiOptimizer, igno
             raise ValueError(
                 "Model already has post_accumulate_grad_hooks. If this is expected, rerun with `ignore_existing_hooks=True`."
             )
-        registered.append(p.register_post_accumulate_grad_hook(partial(_gradient_release_hook, optimizer=optimizer)))
+        registered.append(p.register_post_accumulate_grad_hook(hook))
     model._gradient_release_hooks = registered
+    # the hooks refer to the optimizer weakly; the model keeps it alive, as the reference's hooks do
+    model._gradient_release_optimizer = optimizer
 
 
 def remove_gradient_release(model: Module):
@@ -62,3 +67,5 @@ def remove_gradient_release(model: Module):
     for handle in model._gradient_release_hooks:
         handle.remove()
     del model._gradient_release_hooks
+    if hasattr(model, "_gradient_release_optimizer"):
+        del model._gradient_release_optimizer

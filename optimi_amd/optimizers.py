@@ -51,11 +51,12 @@ class OptimiOptimizer(Optimizer):
     _kahan_placeholder_dtype: torch.dtype | None = torch.uint8  # None: use the parameter dtype (Lion)
     _setup_before_state = False             # StableAdamW resolves its backend before touching state
     _step_state_from_group = True           # per-parameter counter keyed on the group's gradient_release flag (Adan: on the call)
+    _release_kind = ""                      # name of the native hook's optimizer kind (KIND_* of the extension)
 
     # Gradient release parks the steps of tensors with at most this many elements and launches
     # them together when the backward pass ends (0 = launch every tensor on its own, from its
     # hook).  Results are identical; a model with thousands of small tensors steps several times
-    # faster.  Set on the instance, or on the class, before the first backward pass.
+    # faster.  Set on the instance, or on the class, before prepare_for_gradient_release.
     gradient_release_coalesce = 65536
     _QUEUE_MAX_TENSORS = 1024               # parked steps per launch
     _QUEUE_MAX_ELEMENTS = 1 << 24           # parked gradient elements kept alive at most
@@ -89,7 +90,7 @@ class OptimiOptimizer(Optimizer):
         self._optimizer_accumulation = False
         self._hip_groups: dict = {}
         self._release_queue = None
-        self._flush_scheduled = False
+        self._release_hook = None
 
         if self.defaults["gradient_release"]:
             self.defaults["foreach"] = False
@@ -104,14 +105,15 @@ class OptimiOptimizer(Optimizer):
         state = dict(state)
         state.pop("_hip_groups", None)
         state.pop("_release_queue", None)
-        state.pop("_flush_scheduled", None)
+        state.pop("_release_hook", None)
         return state
 
     def __setstate__(self, state):
         super().__setstate__(state)
         self.__dict__.setdefault("_hip_groups", {})
         self.__dict__.setdefault("_release_queue", None)
-        self.__dict__.setdefault("_flush_scheduled", False)
+        self.__dict__.setdefault("_release_hook", None)
+        self._invalidate_release_cache()
         self.__dict__.setdefault("_optimizer_accumulation", False)
 
     def state_dict(self):
@@ -252,23 +254,58 @@ class OptimiOptimizer(Optimizer):
         if not group["triton"]:
             raise RuntimeError("optimi_amd: parameter is not eligible for the HIP backend and there is no other backend")
         backend.check_supported(param)
-        ext = backend.ext()
-        # steps are parked only inside a backward pass, whose end launches them
-        queue = None
-        if self.gradient_release_coalesce > 0 and torch._C._current_graph_task_id() != -1:
-            queue = self._release_queue
-            if queue is None:
-                queue = self._release_queue = ext.ReleaseQueue(self.gradient_release_coalesce, self._QUEUE_MAX_TENSORS,
-                                                               self._QUEUE_MAX_ELEMENTS)
-        parked = self._release_call(ext, group, state, param, param.grad, not self._optimizer_accumulation, queue)
+        parked_or_not = self._release_call(backend.ext(), group, state, param, param.grad, not self._optimizer_accumulation,
+                                           self._queue())
+        del parked_or_not  # the queue itself arranges for its flush at the end of the backward pass
         param.grad = None
-        if parked and not self._flush_scheduled:
-            Variable._execution_engine.queue_callback(self._flush_release)
-            self._flush_scheduled = True
+
+    def _queue(self):
+        """The queue that parks the steps of small tensors during a backward pass, or None."""
+        if self._release_queue is None and self.gradient_release_coalesce > 0:
+            self._release_queue = backend.ext().ReleaseQueue(self.gradient_release_coalesce, self._QUEUE_MAX_TENSORS,
+                                                             self._QUEUE_MAX_ELEMENTS)
+        return self._release_queue
+
+    def _release_entry(self, param: Tensor):
+        """Slow path of the native hook, taken the first time it sees a parameter (and again when
+        the parameter's state was replaced): creates the state as ``step(param=param)`` would and
+        returns ``(state, group, launch workspace or None)``."""
+        state = self.state[param]
+        group = state["group"]
+        if group["triton"] is None:
+            group["triton"] = _default_to_fused([param])
+        self._init_state(group, state, param, True)
+        if not group["triton"]:
+            raise RuntimeError("optimi_amd: parameter is not eligible for the HIP backend and there is no other backend")
+        backend.check_supported(param)
+        return state, group, self._release_workspace(param)
+
+    def _release_workspace(self, param: Tensor):
+        """Hook for subclasses whose per-tensor step needs device scratch."""
+        return None
+
+    def _native_hook(self):
+        """The post-accumulate-grad hook for this optimizer's parameters: a native callable (one
+        per optimizer, shared by its parameters) that does what ``_release`` does."""
+        if self._release_hook is None:
+            ext = backend.ext()
+            self._release_hook = ext.ReleaseHookCore(self, getattr(ext, self._release_kind), self._queue())
+        return backend.ext().ReleaseHook(self._release_hook)
+
+    def _invalidate_release_cache(self):
+        if self.__dict__.get("_release_hook") is not None:
+            self._release_hook.invalidate()
+
+    def load_state_dict(self, state_dict):
+        super().load_state_dict(state_dict)
+        self._invalidate_release_cache()
+
+    def add_param_group(self, param_group):
+        super().add_param_group(param_group)
+        self._invalidate_release_cache()
 
     def _flush_release(self):
         """Launches the gradient-release steps that are still parked."""
-        self._flush_scheduled = False
         if self._release_queue is not None:
             self._release_queue.flush()
 
@@ -322,6 +359,8 @@ class Adam(OptimiOptimizer):
     """
 
     _moment_keys = ("exp_avg", "exp_avg_sq")
+
+    _release_kind = "KIND_ADAM"
 
     def __init__(
         self,
@@ -404,6 +443,8 @@ class Lion(OptimiOptimizer):
     _has_step = False
     _kahan_placeholder_dtype = None
 
+    _release_kind = "KIND_LION"
+
     def __init__(
         self,
         params: Iterable[Tensor] | Iterable[dict],
@@ -464,6 +505,8 @@ class StableAdamW(OptimiOptimizer):
     _moment_keys = ("exp_avg", "exp_avg_sq")
     _setup_before_state = True
 
+    _release_kind = "KIND_STABLEADAMW"
+
     def __init__(
         self,
         params: Iterable[Tensor] | Iterable[dict],
@@ -503,8 +546,11 @@ class StableAdamW(OptimiOptimizer):
                       _groups=self._hip_groups)
 
 
+    def _release_workspace(self, param):
+        return F._workspace(self._hip_groups, param.device, param.dtype, "stableadamw_single")
+
     def _release_call(self, ext, group, state, param, grad, update, queue):
-        grp = F._workspace(self._hip_groups, param.device, param.dtype, "stableadamw_single")
+        grp = self._release_workspace(param)
         return ext.stableadamw_release(grp, param, grad, state["exp_avg"], state["exp_avg_sq"], state["kahan_comp"], state["step"],
                                 group["lr"], group["beta1"], group["beta2"], group["weight_decay"], group["eps"],
                                 group["decouple_lr"], group["max_lr"], bool(group["kahan_sum"]), update, queue)
@@ -530,6 +576,8 @@ class Adan(OptimiOptimizer):
 
     _moment_keys = ("exp_avg", "exp_avg_diff", "exp_avg_sq")
     _step_state_from_group = False
+
+    _release_kind = "KIND_ADAN"
 
     def __init__(
         self,
@@ -601,6 +649,8 @@ class SGD(OptimiOptimizer):
     """
 
     _has_step = False
+
+    _release_kind = "KIND_SGD"
 
     def __init__(
         self,
@@ -674,6 +724,8 @@ class RAdam(OptimiOptimizer):
 
     _moment_keys = ("exp_avg", "exp_avg_sq")
 
+    _release_kind = "KIND_RADAM"
+
     def __init__(
         self,
         params: Iterable[Tensor] | Iterable[dict],
@@ -727,6 +779,8 @@ class Ranger(OptimiOptimizer):
     """
 
     _moment_keys = ("exp_avg", "exp_avg_sq")
+
+    _release_kind = "KIND_RANGER"
 
     def __init__(
         self,

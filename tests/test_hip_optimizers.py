@@ -285,6 +285,62 @@ def test_release_outside_a_backward_pass_launches_at_once(hip_device):
     opt = optimi_amd.AdamW([p], lr=1e-3, gradient_release=True)
     p.grad = torch.full_like(p, 1e-3)
     opt._release(p)
-    assert opt._release_queue is None and p.grad is None
+    assert opt._release_queue.pending() == 0 and p.grad is None
     assert not torch.equal(p.detach(), before)
     assert int(opt.state_dict()["state"][0]["step"]) == 1
+
+
+@pytest.mark.parametrize("case", ["adamw", "lion", "stableadamw", "adan", "sgd", "radam", "ranger"])
+def test_native_hook_equals_python_hook(case, hip_device):
+    """The registered (native) hook against the Python hook body on the same gradients, with a
+    learning-rate change, a state_dict round trip into the live optimizer and a replaced state
+    tensor in between: the native hook re-reads hyper-parameters every call and notices both."""
+    from functools import partial
+
+    from optimi_amd.gradient_release import _gradient_release_hook
+
+    cls, _, hyper = CASES[case]
+    a, b = ManySmall(hip_device), ManySmall(hip_device)
+    native, python = cls(a.parameters(), gradient_release=True, **hyper), cls(b.parameters(), gradient_release=True, **hyper)
+    optimi_amd.prepare_for_gradient_release(a, native)
+    handles = [p.register_post_accumulate_grad_hook(partial(_gradient_release_hook, optimizer=python)) for p in b.parameters()]
+    for it in range(9):
+        native.optimizer_accumulation = python.optimizer_accumulation = it in (1, 2)
+        if it == 3:
+            for opt in (native, python):
+                opt.param_groups[0]["lr"] *= 0.5
+        if it == 5:
+            for opt in (native, python):
+                opt.load_state_dict(opt.state_dict())
+        if it == 7:  # a state tensor replaced behind the optimizer's back
+            for opt, model in ((native, a), (python, b)):
+                st = opt.state[model.ps[4]]
+                st["exp_avg"] = st["exp_avg"].clone().mul_(0.5)
+        for model in (a, b):
+            model(1.0 + it).backward()
+        assert all(p.grad is None for p in a.parameters()) and all(p.grad is None for p in b.parameters())
+    for i, (pa, pb) in enumerate(zip(a.parameters(), b.parameters())):
+        G.assert_bits_equal(pa, pb, f"{case} param {i}")
+        assert list(native.state[pa].keys()) == list(python.state[pb].keys())
+        for key, val in native.state[pa].items():
+            if torch.is_tensor(val) and val.is_cuda and val.is_floating_point():
+                G.assert_bits_equal(val, python.state[pb][key], f"{case} {key} {i}")
+        if "step" in native.state[pa]:
+            assert int(native.state[pa]["step"]) == int(python.state[pb]["step"]) == 9
+    optimi_amd.remove_gradient_release(a)
+    for h in handles:
+        h.remove()
+
+
+def test_hooks_do_not_keep_model_or_optimizer_alive(hip_device):
+    import gc
+    import weakref
+
+    model = ManySmall(hip_device)
+    opt = optimi_amd.AdamW(model.parameters(), lr=1e-3, gradient_release=True)
+    optimi_amd.prepare_for_gradient_release(model, opt)
+    model(1.0).backward()
+    refs = [weakref.ref(model), weakref.ref(opt), weakref.ref(model.ps[0])]
+    del model, opt
+    gc.collect()
+    assert all(r() is None for r in refs)
