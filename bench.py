@@ -16,6 +16,10 @@ the kernel alone: algorithmic bytes per step (each input read once, each output 
 once) over the mean per-step device time between HIP events recorded on the launch stream.
 ``cpu_baseline`` times the PyTorch for-loop restatement (oracle/forloop.py) on this host's
 cores on a bounded sample of the same list.
+
+Two more workloads time gradient release instead (see release_bench):
+``adamw_bf16_kahan_release_stress10k`` (10,000 small tensors, launch-bound) and
+``adamw_bf16_kahan_release_llama7b``; ``--no-coalesce`` turns the parking of small tensors off.
 """
 
 from __future__ import annotations
@@ -129,6 +133,93 @@ def cpu_baseline(cls_name, kwargs, dtype, shapes, budget_s=20.0):
     }
 
 
+def stress_shapes(n_tensors=10_000, lo=128, hi=65536, seed=6):
+    """Sizes log-uniform in [lo, hi]: the many-small-tensors list of the gradient-release stress case."""
+    import math
+
+    import torch
+
+    gen = torch.Generator().manual_seed(seed)
+    u = torch.empty(n_tensors).uniform_(math.log(lo), math.log(hi), generator=gen)
+    return [(int(n),) for n in torch.exp(u).long().clamp(lo, hi).tolist()]
+
+
+def release_bench(args):
+    """Gradient release: AdamW bf16 + Kahan stepped per tensor from real post-accumulate-grad hooks,
+    in cycles of 3 accumulate-only backward passes and 1 full one.  An autograd function hands
+    pre-made gradients to the parameters, so the backward pass launches no kernels of its own and
+    what is timed is the engine's per-parameter work plus the optimizer.  A "step" is one backward
+    pass over the list; the roofline figure counts 48 bytes per parameter per 4-pass cycle."""
+    import torch
+
+    import optimi_amd
+
+    device = torch.device("cuda:0")
+    shapes = stress_shapes() if args.workload.endswith("stress10k") else llama_shapes(4096, 11008, 32)
+    n_params = sum(numel(s) for s in shapes)
+    params = [torch.nn.Parameter(p) for p in make_tensors(shapes, torch.bfloat16, device, 0, 0.02, ones_for_1d=True)]
+    grads = make_tensors(shapes, torch.bfloat16, device, 100, 1e-3)
+    model = torch.nn.Module()
+    model.ps = torch.nn.ParameterList(params)
+
+    class Feed(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, *ps):
+            return ps[0].new_zeros(())
+
+        @staticmethod
+        def backward(ctx, grad_out):
+            return tuple(g.view(g.shape) for g in grads)  # fresh tensor objects, so autograd adopts them as .grad
+
+    # what the same backward pass costs when the hook only frees the gradient: the share of the
+    # autograd engine and of this harness in the figures below
+    handles = [p.register_post_accumulate_grad_hook(lambda p: setattr(p, "grad", None)) for p in params]
+    for _ in range(2):
+        Feed.apply(*params).backward()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(6):
+        Feed.apply(*params).backward()
+    torch.cuda.synchronize()
+    floor_ms = (time.perf_counter() - t0) / 6 * 1e3
+    for h in handles:
+        h.remove()
+
+    kwargs = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
+    opt = optimi_amd.AdamW(params, gradient_release=True, **kwargs)
+    if args.no_coalesce:
+        opt.gradient_release_coalesce = 0
+    optimi_amd.prepare_for_gradient_release(model, opt)
+
+    def one_pass(i):
+        opt.optimizer_accumulation = (i + 1) % 4 != 0
+        Feed.apply(*params).backward()
+
+    for i in range(args.warmup):
+        one_pass(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        one_pass(args.warmup + i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    full = sum(1 for i in range(args.steps) if (args.warmup + i + 1) % 4 == 0)
+    algo_bytes = n_params * (18.0 * full + 10.0 * (args.steps - full))
+    achieved = algo_bytes / elapsed / 1e9
+    print(json.dumps({
+        "metric": "gradient-release tensor-steps/s (AdamW bf16 Kahan, accumulation_steps=4)",
+        "value": len(shapes) * args.steps / elapsed, "unit": "tensor-steps/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "optimizer": "AdamW", "n_tensors": len(shapes), "n_params": n_params,
+                   "coalesce": opt.gradient_release_coalesce, "empty_hook_pass_ms": floor_ms,
+                   "us_per_tensor_over_empty_hook": (elapsed / args.steps * 1e3 - floor_ms) * 1e3 / len(shapes), "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()}},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": None, "note": "wall-clock over whole backward passes, launch-bound for small tensors"},
+        "cpu_baseline": None,
+    }), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -137,6 +228,8 @@ def main():
     ap.add_argument("--workload", default="adamw_bf16_kahan_llama7b")
     ap.add_argument("--grad-sets", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-coalesce", action="store_true",
+                    help="gradient-release workloads: launch every tensor from its own hook instead of parking small ones")
     ap.add_argument("--copy-probe-bytes", type=int, default=0,
                     help="also run the library's plain copy kernel over this many bytes (3 launches) before the "
                          "workload; a profiler run uses it to scale its byte counters against a known size")
@@ -164,6 +257,8 @@ def main():
                        "optimi_hip_copy_probe")
         torch.cuda.synchronize()
         del src, dst
+    if args.workload in ("adamw_bf16_kahan_release_stress10k", "adamw_bf16_kahan_release_llama7b"):
+        return release_bench(args)
     cls_name, kwargs, dtype_name, shapes, bytes_per_param = workloads()[args.workload]
     dtype = getattr(torch, dtype_name)
     n_params = sum(numel(s) for s in shapes)
