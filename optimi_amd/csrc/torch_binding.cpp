@@ -453,6 +453,49 @@ void launch_now(const StepCall& c, Group* stable_group) {
   }
 }
 
+// One whole-list launch of `kind`: ptr[a][i] is tensor i of array a, in the ABI's order for
+// that kind; an array whose first pointer is NULL is passed as absent (Kahan buffers when the
+// Kahan branch is off, SGD's momentum buffer without momentum).
+void launch_list(Kind kind, optimi_group* g, int n, const std::vector<void*>* ptr, const int64_t* numel, int dtype,
+                 const double* s, uint32_t flags, hipStream_t stream) {
+  auto arr = [&](int a) { return (void* const*)ptr[a].data(); };
+  auto carr = [&](int a) { return (const void* const*)ptr[a].data(); };
+  auto opt = [&](int a) { return (n > 0 && ptr[a][0]) ? (void* const*)ptr[a].data() : nullptr; };
+  int rc = 0;
+  const char* what = "";
+  switch (kind) {
+    case ADAM:
+      rc = optimi_hip_adam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], flags, stream);
+      what = "optimi_hip_adam_multi";
+      break;
+    case LION:
+      rc = optimi_hip_lion_multi(g, n, arr(0), carr(1), arr(2), opt(3), numel, dtype, s[0], s[1], s[2], s[3], flags, stream);
+      what = "optimi_hip_lion_multi";
+      break;
+    case STABLEADAMW:
+      rc = optimi_hip_stableadamw_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], flags, stream);
+      what = "optimi_hip_stableadamw_multi";
+      break;
+    case ADAN:
+      rc = optimi_hip_adan_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), arr(5), opt(6), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], flags, stream);
+      what = "optimi_hip_adan_multi";
+      break;
+    case SGD:
+      rc = optimi_hip_sgd_multi(g, n, arr(0), carr(1), opt(2), opt(3), numel, dtype, s[0], s[1], s[2], flags, stream);
+      what = "optimi_hip_sgd_multi";
+      break;
+    case RADAM:
+      rc = optimi_hip_radam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], flags, stream);
+      what = "optimi_hip_radam_multi";
+      break;
+    case RANGER:
+      rc = optimi_hip_ranger_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), opt(5), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], flags, stream);
+      what = "optimi_hip_ranger_multi";
+      break;
+  }
+  check_status(rc, what);
+}
+
 // Parks the steps of small tensors and launches them together, as one list per run of steps
 // that share everything but their tensors (optimizer, dtype, device, stream, flags and every
 // scalar - which includes the step count through the debiased betas).  A tensor of a few
@@ -521,7 +564,6 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
     const StepCall& c0 = batch[0];
     const int n = (int)batch.size(), nt = kTensorsOf[c0.kind];
     const int dtype = dtype_code(c0.param());
-    const bool kahan = c0.kahan().has_value();
     std::vector<void*> ptr[kMaxTensors];
     std::vector<int64_t> numel((size_t)n);
     for (int a = 0; a < nt; ++a) ptr[a].resize((size_t)n, nullptr);
@@ -530,47 +572,10 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
       for (int a = 0; a < nt; ++a)
         if (batch[(size_t)i].t[a].has_value()) ptr[a][(size_t)i] = batch[(size_t)i].t[a]->data_ptr();
     }
-    auto arr = [&](int a) { return (void* const*)ptr[a].data(); };
-    auto carr = [&](int a) { return (const void* const*)ptr[a].data(); };
-    auto opt = [&](int a, bool present) { return present ? (void* const*)ptr[a].data() : nullptr; };
-    const double* s = c0.s;
     c10::hip::HIPGuardMasqueradingAsCUDA guard(c0.param().device());
     std::unique_ptr<Group>& slot = groups_[c0.param().device().index()];  // a workspace lives on one device
     if (!slot) slot = std::make_unique<Group>();  // made on first use: a queue may exist before any device work
-    optimi_group* g = slot->get();
-    int rc = 0;
-    const char* what = "";
-    switch (c0.kind) {
-      case ADAM:
-        rc = optimi_hip_adam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], c0.flags, stream_);
-        what = "optimi_hip_adam_multi";
-        break;
-      case LION:
-        rc = optimi_hip_lion_multi(g, n, arr(0), carr(1), arr(2), opt(3, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], c0.flags, stream_);
-        what = "optimi_hip_lion_multi";
-        break;
-      case STABLEADAMW:
-        rc = optimi_hip_stableadamw_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], c0.flags, stream_);
-        what = "optimi_hip_stableadamw_multi";
-        break;
-      case ADAN:
-        rc = optimi_hip_adan_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), arr(5), opt(6, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], c0.flags, stream_);
-        what = "optimi_hip_adan_multi";
-        break;
-      case SGD:
-        rc = optimi_hip_sgd_multi(g, n, arr(0), carr(1), opt(2, c0.t[2].has_value()), opt(3, kahan), numel.data(), dtype, s[0], s[1], s[2], c0.flags, stream_);
-        what = "optimi_hip_sgd_multi";
-        break;
-      case RADAM:
-        rc = optimi_hip_radam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], c0.flags, stream_);
-        what = "optimi_hip_radam_multi";
-        break;
-      case RANGER:
-        rc = optimi_hip_ranger_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), opt(5, kahan), numel.data(), dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], c0.flags, stream_);
-        what = "optimi_hip_ranger_multi";
-        break;
-    }
-    check_status(rc, what);
+    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtype, c0.s, c0.flags, stream_);
   }
 
  private:
@@ -616,68 +621,116 @@ bool submit(StepCall&& c, ReleaseQueue* queue, Group* stable_group = nullptr) {
   return false;
 }
 
+// The scalar prologue of each functional form: flags and scalars as the ABI takes them, from
+// the raw hyper-parameters and the step count `t` (1-based, already advanced).
+struct Hyper {
+  uint32_t flags = 0;
+  double s[kMaxScalars] = {0, 0, 0, 0, 0, 0, 0, 0};
+};
+
+double decayed(double weight_decay, double lr, bool decouple_wd, bool decouple_lr, const std::optional<double>& max_lr) {
+  if (weight_decay == 0) return 0;
+  if (decouple_lr) return 1 - (lr / max_lr.value()) * weight_decay;
+  if (decouple_wd) return 1 - lr * weight_decay;
+  return weight_decay;  // L2: the raw coefficient
+}
+
+Hyper adam_hyper(int64_t t, double lr, double beta1, double beta2, double weight_decay, double eps, bool decouple_wd,
+                 bool decouple_lr, const std::optional<double>& max_lr, bool kahan_sum, bool update) {  // optimi/adam.py:260-273
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
+  return {base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u),
+          {lr, 1 - b1h, b2h, 1 - b2h, decayed(weight_decay, lr, decouple_wd, decouple_lr, max_lr), eps}};
+}
+
+Hyper lion_hyper(double lr, double beta1, double beta2, double weight_decay, bool decouple_lr,
+                 const std::optional<double>& max_lr, bool kahan_sum, bool update) {  // optimi/lion.py:226-235
+  return {base_flags(kahan_sum, update), {lr, 1 - beta1, 1 - beta2, decayed(weight_decay, lr, true, decouple_lr, max_lr)}};
+}
+
+Hyper stableadamw_hyper(int64_t t, double lr, double beta1, double beta2, double weight_decay, double eps, bool decouple_lr,
+                        const std::optional<double>& max_lr, bool kahan_sum, bool update) {  // optimi/stableadamw.py:326-332
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
+  return {base_flags(kahan_sum, update) | (decouple_lr ? OPTIMI_DECOUPLE_LR : 0u),
+          {lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps, (decouple_lr && max_lr.has_value()) ? *max_lr : 0.0}};
+}
+
+Hyper adan_hyper(int64_t t, double lr, double beta1, double beta2, double beta3, double weight_decay, double eps,
+                 bool decouple_lr, const std::optional<double>& max_lr, bool adam_wd, bool kahan_sum, bool update) {  // optimi/adan.py:289-309
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t), b3h = debias_beta(beta3, t);
+  if (weight_decay != 0) {
+    weight_decay = decouple_lr ? (lr / max_lr.value()) * weight_decay : lr * weight_decay;
+    weight_decay = adam_wd ? 1 - weight_decay : 1 + weight_decay;
+  }
+  return {base_flags(kahan_sum, update) | (adam_wd ? OPTIMI_ADAM_WD : 0u),
+          {lr, 1 - b1h, beta2, 1 - b2h, b3h, 1 - b3h, eps, weight_decay}};
+}
+
+Hyper sgd_hyper(double lr, double momentum, double weight_decay, bool dampening, bool decouple_wd, bool decouple_lr,
+                const std::optional<double>& max_lr, bool kahan_sum, bool update) {  // optimi/sgd.py:213-240
+  return {base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u) | (dampening ? OPTIMI_DAMPENING : 0u),
+          {lr, momentum, decayed(weight_decay, lr, decouple_wd, decouple_lr, max_lr)}};
+}
+
+// RAdam (optimi/radam.py:214-322) and, with lookahead, Ranger (optimi/ranger.py:230-344)
+Hyper ranger_hyper(int64_t t, bool lookahead, double lr, double beta1, double beta2, double weight_decay, double eps,
+                   int64_t sync_every, double alpha, bool decouple_wd, bool decouple_lr, const std::optional<double>& max_lr,
+                   bool kahan_sum, bool update) {
+  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
+  const double rect = rectification(beta2, t);
+  uint32_t flags = base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u) |
+                   (rect >= 0 ? OPTIMI_RECTIFY : 0u);
+  if (lookahead && t % sync_every == 0) flags |= OPTIMI_LOOKAHEAD;
+  return {flags, {lr, 1 - b1h, b2h, 1 - b2h, decayed(weight_decay, lr, decouple_wd, decouple_lr, max_lr), eps,
+                  rect >= 0 ? rect : 0.0, alpha}};
+}
+
+StepCall make_call(Kind kind, const Hyper& h, std::initializer_list<std::optional<at::Tensor>> tensors) {
+  StepCall c;
+  c.kind = kind;
+  c.flags = h.flags;
+  std::memcpy(c.s, h.s, sizeof(c.s));
+  int a = 0;
+  for (const auto& t : tensors) c.t[a++] = t;
+  return c;
+}
+
 bool adam_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
                   const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
                   double weight_decay, double eps, bool decouple_wd, bool decouple_lr, std::optional<double> max_lr,
                   bool kahan_sum, bool update, ReleaseQueue* queue) {
-  const int64_t t = tick(step);
-  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
-  if (weight_decay != 0) {
-    if (decouple_lr) weight_decay = 1 - (lr / max_lr.value()) * weight_decay;
-    else if (decouple_wd) weight_decay = 1 - lr * weight_decay;
-  }
-  StepCall c{ADAM, base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u),
-             {p, grad_like(p, g), m, v, real_kahan(p, k)}, {lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps}};
-  return submit(std::move(c), queue);
+  const Hyper h = adam_hyper(tick(step), lr, beta1, beta2, weight_decay, eps, decouple_wd, decouple_lr, max_lr, kahan_sum, update);
+  return submit(make_call(ADAM, h, {p, grad_like(p, g), m, v, real_kahan(p, k)}), queue);
 }
 
 bool lion_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const std::optional<at::Tensor>& k,
                   double lr, double beta1, double beta2, double weight_decay, bool decouple_lr,
                   std::optional<double> max_lr, bool kahan_sum, bool update, ReleaseQueue* queue) {
-  if (weight_decay != 0) weight_decay = decouple_lr ? 1 - (lr / max_lr.value()) * weight_decay : 1 - lr * weight_decay;
-  StepCall c{LION, base_flags(kahan_sum, update), {p, grad_like(p, g), m, real_kahan(p, k)}, {lr, 1 - beta1, 1 - beta2, weight_decay}};
-  return submit(std::move(c), queue);
+  const Hyper h = lion_hyper(lr, beta1, beta2, weight_decay, decouple_lr, max_lr, kahan_sum, update);
+  return submit(make_call(LION, h, {p, grad_like(p, g), m, real_kahan(p, k)}), queue);
 }
 
 bool stableadamw_release(Group& group, const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
                          const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
                          double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum,
                          bool update, ReleaseQueue* queue) {
-  const int64_t t = tick(step);
-  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
-  StepCall c{STABLEADAMW, base_flags(kahan_sum, update) | (decouple_lr ? OPTIMI_DECOUPLE_LR : 0u),
-             {p, grad_like(p, g), m, v, real_kahan(p, k)},
-             {lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps, (decouple_lr && max_lr.has_value()) ? *max_lr : 0.0}};
-  return submit(std::move(c), queue, &group);
+  const Hyper h = stableadamw_hyper(tick(step), lr, beta1, beta2, weight_decay, eps, decouple_lr, max_lr, kahan_sum, update);
+  return submit(make_call(STABLEADAMW, h, {p, grad_like(p, g), m, v, real_kahan(p, k)}), queue, &group);
 }
 
 bool adan_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& df, const at::Tensor& n,
                   const at::Tensor& pg, const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1,
                   double beta2, double beta3, double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr,
                   bool adam_wd, bool kahan_sum, bool update, ReleaseQueue* queue) {
-  const int64_t t = tick(step);
-  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t), b3h = debias_beta(beta3, t);
-  if (weight_decay != 0) {
-    weight_decay = decouple_lr ? (lr / max_lr.value()) * weight_decay : lr * weight_decay;
-    weight_decay = adam_wd ? 1 - weight_decay : 1 + weight_decay;
-  }
-  StepCall c{ADAN, base_flags(kahan_sum, update) | (adam_wd ? OPTIMI_ADAM_WD : 0u),
-             {p, grad_like(p, g), m, df, n, pg, real_kahan(p, k)},
-             {lr, 1 - b1h, beta2, 1 - b2h, b3h, 1 - b3h, eps, weight_decay}};
-  return submit(std::move(c), queue);
+  const Hyper h = adan_hyper(tick(step), lr, beta1, beta2, beta3, weight_decay, eps, decouple_lr, max_lr, adam_wd, kahan_sum, update);
+  return submit(make_call(ADAN, h, {p, grad_like(p, g), m, df, n, pg, real_kahan(p, k)}), queue);
 }
 
 bool sgd_release(const at::Tensor& p, const at::Tensor& g, const std::optional<at::Tensor>& m,
                  const std::optional<at::Tensor>& k, double lr, double momentum, double weight_decay, bool dampening,
                  bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update,
                  ReleaseQueue* queue) {
-  if (weight_decay != 0) {
-    if (decouple_lr) weight_decay = 1 - (lr / max_lr.value()) * weight_decay;
-    else if (decouple_wd) weight_decay = 1 - lr * weight_decay;
-  }
-  StepCall c{SGD, base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u) | (dampening ? OPTIMI_DAMPENING : 0u),
-             {p, grad_like(p, g), momentum != 0 ? real_kahan(p, m) : std::nullopt, real_kahan(p, k)}, {lr, momentum, weight_decay}};
-  return submit(std::move(c), queue);
+  const Hyper h = sgd_hyper(lr, momentum, weight_decay, dampening, decouple_wd, decouple_lr, max_lr, kahan_sum, update);
+  return submit(make_call(SGD, h, {p, grad_like(p, g), momentum != 0 ? real_kahan(p, m) : std::nullopt, real_kahan(p, k)}), queue);
 }
 
 bool ranger_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
@@ -685,24 +738,11 @@ bool ranger_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& 
                     double beta1, double beta2, double weight_decay, double eps, int64_t sync_every, double alpha,
                     bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update,
                     ReleaseQueue* queue) {
-  // la = None makes this RAdam (optimi/radam.py:214-322); with la it is Ranger (optimi/ranger.py:230-344)
-  const int64_t t = tick(step);
-  const double b1h = debias_beta(beta1, t), b2h = debias_beta(beta2, t);
-  const double rect = rectification(beta2, t);
-  if (weight_decay != 0) {
-    if (decouple_lr) weight_decay = 1 - (lr / max_lr.value()) * weight_decay;
-    else if (decouple_wd) weight_decay = 1 - lr * weight_decay;
-  }
-  uint32_t flags = base_flags(kahan_sum, update) | ((decouple_wd || decouple_lr) ? OPTIMI_DECOUPLE_WD : 0u) |
-                   (rect >= 0 ? OPTIMI_RECTIFY : 0u);
-  const double r = rect >= 0 ? rect : 0.0;
-  if (la.has_value()) {
-    if (t % sync_every == 0) flags |= OPTIMI_LOOKAHEAD;
-    StepCall c{RANGER, flags, {p, grad_like(p, g), m, v, *la, real_kahan(p, k)}, {lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps, r, alpha}};
-    return submit(std::move(c), queue);
-  }
-  StepCall c{RADAM, flags, {p, grad_like(p, g), m, v, real_kahan(p, k)}, {lr, 1 - b1h, b2h, 1 - b2h, weight_decay, eps, r}};
-  return submit(std::move(c), queue);
+  // la = None makes this RAdam; with la it is Ranger
+  const Hyper h = ranger_hyper(tick(step), la.has_value(), lr, beta1, beta2, weight_decay, eps, sync_every, alpha, decouple_wd,
+                               decouple_lr, max_lr, kahan_sum, update);
+  if (la.has_value()) return submit(make_call(RANGER, h, {p, grad_like(p, g), m, v, *la, real_kahan(p, k)}), queue);
+  return submit(make_call(RADAM, h, {p, grad_like(p, g), m, v, real_kahan(p, k)}), queue);
 }
 
 
@@ -742,6 +782,7 @@ class ReleaseHookCore {
     rebind();
   }
 
+
   void call(const py::handle& param_h) {
     TORCH_CHECK(THPVariable_Check(param_h.ptr()), "optimi_amd: the gradient release hook takes the parameter");
     py::object optimizer = optimizer_();
@@ -752,52 +793,91 @@ class ReleaseHookCore {
     }
     const at::Tensor& p = THPVariable_Unpack(param_h.ptr());
     Entry* e = find(p);
-    if (!e || !valid(*e)) e = refresh(optimizer, param_h, p);
+    if (!e || !valid(*e)) e = refresh(optimizer, k_.entry, param_h, p, true);
     const at::Tensor g = p.grad();
     TORCH_CHECK(g.defined(), "optimi_amd: the gradient release hook ran on a parameter without a gradient");
     at::NoGradGuard no_grad;
     const bool update = !truthy(py::reinterpret_steal<py::object>(attr(optimizer.ptr(), k_.accumulation)).ptr());
     PyObject* grp = e->group.ptr();
-    ReleaseQueue* q = queue_.get();
-    const auto& t = e->t;
-    switch (kind_) {
-      case ADAM:
-        adam_release(p, g, *t[0], *t[1], t[2], e->step, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2),
-                     num(grp, k_.weight_decay), num(grp, k_.eps), flag(grp, k_.decouple_wd), flag(grp, k_.decouple_lr),
-                     opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update, q);
-        break;
-      case LION:
-        lion_release(p, g, *t[0], t[1], num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2), num(grp, k_.weight_decay),
-                     flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update, q);
-        break;
-      case STABLEADAMW:
-        stableadamw_release(*e->workspace, p, g, *t[0], *t[1], t[2], e->step, num(grp, k_.lr), num(grp, k_.beta1),
-                            num(grp, k_.beta2), num(grp, k_.weight_decay), num(grp, k_.eps), flag(grp, k_.decouple_lr),
-                            opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update, q);
-        break;
-      case ADAN:  // adam_wd is not forwarded by the reference's class either (optimi/adan.py:186-208)
-        adan_release(p, g, *t[0], *t[1], *t[2], *t[3], t[4], e->step, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2),
-                     num(grp, k_.beta3), num(grp, k_.weight_decay), num(grp, k_.eps), flag(grp, k_.decouple_lr),
-                     opt_num(grp, k_.max_lr), false, flag(grp, k_.kahan_sum), update, q);
-        break;
-      case SGD:
-        sgd_release(p, g, t[0], t[1], num(grp, k_.lr), num(grp, k_.momentum), num(grp, k_.weight_decay),
-                    flag(grp, k_.dampening), flag(grp, k_.decouple_wd), flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr),
-                    flag(grp, k_.kahan_sum), update, q);
-        break;
-      case RADAM:
-        ranger_release(p, g, *t[0], *t[1], std::nullopt, t[2], e->step, num(grp, k_.lr), num(grp, k_.beta1),
-                       num(grp, k_.beta2), num(grp, k_.weight_decay), num(grp, k_.eps), 1, 0.0, flag(grp, k_.decouple_wd),
-                       flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update, q);
-        break;
-      case RANGER:
-        ranger_release(p, g, *t[0], *t[1], t[2], t[3], e->step, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2),
-                       num(grp, k_.weight_decay), num(grp, k_.eps), (int64_t)num(grp, k_.k), num(grp, k_.alpha),
-                       flag(grp, k_.decouple_wd), flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr),
-                       flag(grp, k_.kahan_sum), update, q);
-        break;
-    }
+    const Hyper h = read_hyper(grp, has_step_ ? tick(e->step) : 0, update);
+    submit(pack(*e, h, p, grad_like(p, g), num_or_zero(grp)), queue_.get(), e->workspace);
     p.mutable_grad().reset();  // param.grad = None
+  }
+
+  // One whole-group step (optimi/adam.py:158-182 and the functional form behind it) without the
+  // per-parameter Python walk: collects the parameters of `group` that have a gradient, advances
+  // the group's step counter, forms the scalars and launches one list per (device, dtype).
+  // Returns false, having done nothing, when the group has not been set up yet (the first step
+  // goes through Python, which resolves the backend) - the caller then takes the Python path.
+  bool step_group(const py::dict& group) {
+    PyObject* grp = group.ptr();
+    if (!flag(grp, k_.setup) || item(grp, k_.triton) != Py_True) return false;
+    py::object optimizer = optimizer_();
+    TORCH_CHECK(!optimizer.is_none(), "optimi_amd: the optimizer no longer exists");
+    PyObject* plist = item(grp, k_.params);
+    TORCH_CHECK(PyList_Check(plist), "optimi_amd: group['params'] must be a list");
+    at::NoGradGuard no_grad;
+
+    // pass 1: the parameters that step, their cached states (created on first sight); no side effects on steps
+    struct Item {
+      at::Tensor p, g;
+      Entry* e;
+    };
+    std::vector<Item> items;
+    const Py_ssize_t n_params = PyList_GET_SIZE(plist);
+    items.reserve((size_t)n_params);
+    for (Py_ssize_t i = 0; i < n_params; ++i) {
+      PyObject* obj = PyList_GET_ITEM(plist, i);
+      TORCH_CHECK(THPVariable_Check(obj), "optimi_amd: group['params'] holds something that is not a tensor");
+      const at::Tensor& p = THPVariable_Unpack(obj);
+      const at::Tensor& g = p.grad();
+      if (!g.defined()) continue;
+      TORCH_CHECK(!g.is_sparse(), "optimi_amd does not support sparse gradients");
+      Entry* e = find(p);
+      if (!e || !valid(*e, false)) e = refresh(optimizer, k_.group_entry, py::handle(obj), p, false, group);
+      check_param(p);
+      items.push_back({p, grad_like(p, g), e});
+    }
+
+    // the group's counter advances even when nothing has a gradient, as in the reference
+    int64_t t = 0;
+    if (has_step_) {
+      PyObject* step = item(grp, k_.step);
+      TORCH_CHECK(THPVariable_Check(step), "optimi_amd: group['step'] must be a tensor");
+      t = tick(THPVariable_Unpack(step));
+    }
+    if (items.empty()) return true;
+    const Hyper h = read_hyper(grp, t, true);
+    const double momentum = num_or_zero(grp);
+
+    // pass 2: one launch per (device, dtype), in order of first appearance
+    const int nt = kTensorsOf[kind_];
+    std::vector<char> done(items.size(), 0);
+    for (size_t first = 0; first < items.size(); ++first) {
+      if (done[first]) continue;
+      const at::Tensor& p0 = items[first].p;
+      std::vector<void*> ptr[kMaxTensors];
+      std::vector<int64_t> numel;
+      for (size_t i = first; i < items.size(); ++i) {
+        const at::Tensor& p = items[i].p;
+        if (done[i] || p.scalar_type() != p0.scalar_type() || p.device() != p0.device()) continue;
+        done[i] = 1;
+        const StepCall c = pack(*items[i].e, h, p, items[i].g, momentum);
+        for (int a = 1; a < nt; ++a)
+          if (c.t[a].has_value()) check_like(p, *c.t[a], a == 1 ? "grad" : "state");
+        for (int a = 0; a < nt; ++a) ptr[a].push_back(c.t[a].has_value() ? c.t[a]->data_ptr() : nullptr);
+        numel.push_back(p.numel());
+      }
+      // an absent array must be absent for every tensor of the launch
+      for (int a = 2; a < nt; ++a)
+        for (void* q : ptr[a]) TORCH_CHECK((q == nullptr) == (ptr[a][0] == nullptr), "optimi_amd: a state buffer is missing for some parameters of a group");
+      c10::hip::HIPGuardMasqueradingAsCUDA guard(p0.device());
+      std::unique_ptr<Group>& slot = workspaces_[{(int)p0.device().index(), (int)p0.scalar_type()}];
+      if (!slot) slot = std::make_unique<Group>();
+      launch_list(kind_, slot->get(), (int)numel.size(), ptr, numel.data(), dtype_code(p0), h.s, h.flags,
+                  c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(p0.device().index()).stream());
+    }
+    return true;
   }
 
  private:
@@ -807,6 +887,7 @@ class ReleaseHookCore {
     Group* workspace = nullptr;
     PyObject* ids[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
     PyObject* step_id = nullptr;
+    bool release = false;  // made for the gradient-release hook (group and step counter cached too)
     std::optional<at::Tensor> t[5];
     at::Tensor step;
     explicit Entry(const at::Tensor& p) : param(p.getIntrusivePtr()) {}
@@ -817,6 +898,7 @@ class ReleaseHookCore {
     py::str lr{"lr"}, beta1{"beta1"}, beta2{"beta2"}, beta3{"beta3"}, weight_decay{"weight_decay"}, eps{"eps"};
     py::str decouple_wd{"decouple_wd"}, decouple_lr{"decouple_lr"}, max_lr{"max_lr"}, kahan_sum{"kahan_sum"};
     py::str momentum{"momentum"}, dampening{"dampening"}, k{"k"}, alpha{"alpha"};
+    py::str setup{"setup"}, triton{"triton"}, params{"params"}, group_entry{"_group_entry"};
   };
 
   static PyObject* attr(PyObject* obj, const py::str& name) {
@@ -850,6 +932,55 @@ class ReleaseHookCore {
     return as_double(v);
   }
 
+  // SGD keeps a momentum buffer in its state even when momentum is 0; it is not passed then
+  double num_or_zero(PyObject* grp) const { return kind_ == SGD ? num(grp, k_.momentum) : 1.0; }
+
+  Hyper read_hyper(PyObject* grp, int64_t t, bool update) const {
+    switch (kind_) {
+      case ADAM:
+        return adam_hyper(t, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2), num(grp, k_.weight_decay), num(grp, k_.eps),
+                          flag(grp, k_.decouple_wd), flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update);
+      case LION:
+        return lion_hyper(num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2), num(grp, k_.weight_decay),
+                          flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update);
+      case STABLEADAMW:
+        return stableadamw_hyper(t, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2), num(grp, k_.weight_decay),
+                                 num(grp, k_.eps), flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update);
+      case ADAN:  // adam_wd is not forwarded by the reference's class either (optimi/adan.py:186-208)
+        return adan_hyper(t, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2), num(grp, k_.beta3), num(grp, k_.weight_decay),
+                          num(grp, k_.eps), flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), false, flag(grp, k_.kahan_sum), update);
+      case SGD:
+        return sgd_hyper(num(grp, k_.lr), num(grp, k_.momentum), num(grp, k_.weight_decay), flag(grp, k_.dampening),
+                         flag(grp, k_.decouple_wd), flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update);
+      case RADAM:
+        return ranger_hyper(t, false, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2), num(grp, k_.weight_decay),
+                            num(grp, k_.eps), 1, 0.0, flag(grp, k_.decouple_wd), flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr),
+                            flag(grp, k_.kahan_sum), update);
+      case RANGER:
+        return ranger_hyper(t, true, num(grp, k_.lr), num(grp, k_.beta1), num(grp, k_.beta2), num(grp, k_.weight_decay),
+                            num(grp, k_.eps), (int64_t)num(grp, k_.k), num(grp, k_.alpha), flag(grp, k_.decouple_wd),
+                            flag(grp, k_.decouple_lr), opt_num(grp, k_.max_lr), flag(grp, k_.kahan_sum), update);
+    }
+    TORCH_CHECK(false, "optimi_amd: unknown optimizer kind");
+  }
+
+  // The step of one parameter in the ABI's tensor order: param, grad, the states, the Kahan buffer last.
+  StepCall pack(const Entry& e, const Hyper& h, const at::Tensor& p, const at::Tensor& g, double momentum) const {
+    StepCall c;
+    c.kind = kind_;
+    c.flags = h.flags;
+    std::memcpy(c.s, h.s, sizeof(c.s));
+    c.t[0] = p;
+    c.t[1] = g;
+    const size_t n = state_keys_.size();
+    for (size_t i = 0; i < n; ++i) {
+      const bool placeholder_possible = i + 1 == n || kind_ == SGD;  // Kahan buffer; SGD's momentum buffer
+      c.t[2 + i] = placeholder_possible ? real_kahan(p, e.t[i]) : e.t[i];
+    }
+    if (kind_ == SGD && momentum == 0) c.t[2] = std::nullopt;
+    return c;
+  }
+
   void rebind() {
     hook_tables_.clear();
     py::object optimizer = optimizer_();
@@ -881,26 +1012,31 @@ class ReleaseHookCore {
   }
 
   // every cached tensor is still the object the state dict holds
-  bool valid(const Entry& e) const {
+  // (`release`: also the group and the per-parameter step counter that gradient release keeps there)
+  bool valid(const Entry& e, bool release = true) const {
     PyObject* st = e.state.ptr();
     for (size_t i = 0; i < state_keys_.size(); ++i)
       if (PyDict_GetItemWithError(st, state_keys_[i].ptr()) != e.ids[i]) return false;
+    if (!release) return true;
+    if (!e.release) return false;
     if (PyDict_GetItemWithError(st, k_.group.ptr()) != e.group.ptr()) return false;
     if (has_step_ && PyDict_GetItemWithError(st, k_.step.ptr()) != e.step_id) return false;
     return true;
   }
 
-  Entry* refresh(const py::object& optimizer, const py::handle& param_h, const at::Tensor& p) {
+  Entry* refresh(const py::object& optimizer, const py::str& method, const py::handle& param_h, const at::Tensor& p,
+                 bool release, const py::handle& group = py::handle()) {
     PyErr_Clear();
     // (state dict, group dict, launch workspace or None), state created and the backend checked
-    py::tuple made = optimizer.attr(k_.entry)(param_h);
+    py::tuple made = group ? optimizer.attr(method)(param_h, group) : optimizer.attr(method)(param_h);
     Entry e(p);
+    e.release = release;
     e.state = made[0];
     e.group = made[1];
     e.workspace_obj = made[2];
     TORCH_CHECK(PyDict_Check(e.state.ptr()) && PyDict_Check(e.group.ptr()), "optimi_amd: state and group must be dicts");
     if (!e.workspace_obj.is_none()) e.workspace = &e.workspace_obj.cast<Group&>();
-    TORCH_CHECK(kind_ != STABLEADAMW || e.workspace, "optimi_amd: StableAdamW needs a launch workspace");
+    TORCH_CHECK(kind_ != STABLEADAMW || e.workspace || !release, "optimi_amd: StableAdamW needs a launch workspace");
     for (size_t i = 0; i < state_keys_.size(); ++i) {
       PyObject* v = PyDict_GetItemWithError(e.state.ptr(), state_keys_[i].ptr());
       TORCH_CHECK(v, "optimi_amd: optimizer state has no '", std::string(state_keys_[i]), "'");
@@ -913,7 +1049,7 @@ class ReleaseHookCore {
     // all but the last key (the Kahan buffer) and SGD's momentum buffer must be tensors
     for (size_t i = 0; i + 1 < state_keys_.size(); ++i)
       TORCH_CHECK(e.t[i].has_value() || kind_ == SGD, "optimi_amd: state '", std::string(state_keys_[i]), "' is None");
-    if (has_step_) {
+    if (has_step_ && release) {
       PyObject* v = PyDict_GetItemWithError(e.state.ptr(), k_.step.ptr());
       TORCH_CHECK(v && THPVariable_Check(v), "optimi_amd: the per-parameter step counter is missing");
       e.step_id = v;
@@ -931,6 +1067,10 @@ class ReleaseHookCore {
   std::vector<py::str> state_keys_;
   std::vector<py::object> hook_tables_;
   std::unordered_map<c10::TensorImpl*, Entry> entries_;
+  struct PairHash {
+    size_t operator()(const std::pair<int, int>& k) const { return std::hash<int64_t>()(((int64_t)k.first << 32) ^ (int64_t)k.second); }
+  };
+  std::unordered_map<std::pair<int, int>, std::unique_ptr<Group>, PairHash> workspaces_;  // (device, dtype) -> tables
 };
 
 // What is registered on the parameters: a handle that does not own the hook, so that
@@ -966,6 +1106,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   py::class_<ReleaseHookCore, std::shared_ptr<ReleaseHookCore>>(mod, "ReleaseHookCore")
       .def(py::init<const py::object&, int, std::shared_ptr<ReleaseQueue>>(), py::arg("optimizer"), py::arg("kind"), py::arg("queue"))
       .def("invalidate", &ReleaseHookCore::invalidate)
+      .def("step_group", &ReleaseHookCore::step_group)
       .def("__call__", &ReleaseHookCore::call);
   py::class_<ReleaseHook>(mod, "ReleaseHook")
       .def(py::init<const std::shared_ptr<ReleaseHookCore>&>())

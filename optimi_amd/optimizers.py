@@ -57,6 +57,7 @@ class OptimiOptimizer(Optimizer):
     # them together when the backward pass ends (0 = launch every tensor on its own, from its
     # hook).  Results are identical; a model with thousands of small tensors steps several times
     # faster.  Set on the instance, or on the class, before prepare_for_gradient_release.
+    native_step = True                      # False: walk the parameters in Python on every step (same results)
     gradient_release_coalesce = 65536
     _QUEUE_MAX_TENSORS = 1024               # parked steps per launch
     _QUEUE_MAX_ELEMENTS = 1 << 24           # parked gradient elements kept alive at most
@@ -185,7 +186,6 @@ class OptimiOptimizer(Optimizer):
     def _functional(self, group, params, grads, states, step, gradient_release, accumulate):
         raise NotImplementedError
 
-    @torch.no_grad()
     def step(self, closure: Callable | None = None, param: Tensor | None = None):
         """Performs a single optimization step on the whole model or individual parameter.
 
@@ -196,6 +196,19 @@ class OptimiOptimizer(Optimizer):
                 pass. Requires optimizer to be initialized with `gradient_release=True` and model
                 hooks created with `prepare_for_gradient_release`. Incompatible with `closure`.
         """
+        # torch wraps an optimizer's step in a profiler range that runs the step hooks; on a small
+        # model that wrapper costs more than the launch.  It is entered here only when it has
+        # something to do (a hook is registered, or a profiler is recording).
+        if self._has_step_hooks() or torch._C._autograd._profiler_enabled():
+            return self._step_with_hooks(closure=closure, param=param)
+        loss = self._step(closure=closure, param=param)
+        self._optimizer_step_code()
+        return loss
+
+    step.hooked = True  # tells torch.optim.Optimizer not to wrap step() itself
+
+    @torch.no_grad()
+    def _step(self, closure: Callable | None = None, param: Tensor | None = None):
         loss = None
         if closure is not None and param is None:
             with torch.enable_grad():
@@ -203,7 +216,11 @@ class OptimiOptimizer(Optimizer):
 
         if param is None:
             self._flush_release()
+            driver = self._driver() if self.native_step else None
             for group in self.param_groups:
+                # after a group's first step the whole walk over its parameters is native
+                if driver is not None and group["setup"] and driver.step_group(group):
+                    continue
                 params = self._collect(group)
                 if params and not group["triton"]:
                     raise RuntimeError(
@@ -222,6 +239,8 @@ class OptimiOptimizer(Optimizer):
                 raise RuntimeError("optimi_amd: parameter is not eligible for the HIP backend and there is no other backend")
             self._functional(group, param, param.grad, state, state.get("step"), True, self._optimizer_accumulation)
         return loss
+
+    _step_with_hooks = Optimizer.profile_hook_step(_step)
 
     # -- gradient-release fast path --------------------------------------------------------
     def _release_call(self, ext, group, state, param, grad, update, queue):
@@ -280,17 +299,31 @@ class OptimiOptimizer(Optimizer):
         backend.check_supported(param)
         return state, group, self._release_workspace(param)
 
+    def _group_entry(self, param: Tensor, group: dict):
+        """Slow path of the native whole-group step, taken the first time it sees a parameter with
+        a gradient (and again when its state was replaced): creates the state as ``_collect``
+        would and returns ``(state, group, None)``."""
+        state = self.state[param]
+        self._init_state(group, state, param)
+        backend.check_supported(param)
+        return state, group, None
+
     def _release_workspace(self, param: Tensor):
         """Hook for subclasses whose per-tensor step needs device scratch."""
         return None
 
-    def _native_hook(self):
-        """The post-accumulate-grad hook for this optimizer's parameters: a native callable (one
-        per optimizer, shared by its parameters) that does what ``_release`` does."""
+    def _driver(self):
+        """The native driver of this optimizer: the gradient-release hook body and the
+        whole-group step, with their per-parameter cache."""
         if self._release_hook is None:
             ext = backend.ext()
             self._release_hook = ext.ReleaseHookCore(self, getattr(ext, self._release_kind), self._queue())
-        return backend.ext().ReleaseHook(self._release_hook)
+        return self._release_hook
+
+    def _native_hook(self):
+        """The post-accumulate-grad hook for this optimizer's parameters: a native callable (one
+        per optimizer, shared by its parameters) that does what ``_release`` does."""
+        return backend.ext().ReleaseHook(self._driver())
 
     def _invalidate_release_cache(self):
         if self.__dict__.get("_release_hook") is not None:

@@ -344,3 +344,79 @@ def test_hooks_do_not_keep_model_or_optimizer_alive(hip_device):
     del model, opt
     gc.collect()
     assert all(r() is None for r in refs)
+
+
+@pytest.mark.parametrize("case", list(CASES))
+def test_native_group_step_equals_python_walk(case, hip_device):
+    """step() with the parameter walk in native code against the Python walk (native_step=False):
+    two groups, two dtypes, parameters whose gradient is missing on some steps or arrives late,
+    a learning-rate change, a state_dict round trip into the live optimizer, a replaced state
+    tensor, and a step on which nothing has a gradient (the step counter still advances)."""
+    cls, _, hyper = CASES[case]
+    a, b = ManySmall(hip_device), ManySmall(hip_device)
+
+    def build(model):
+        ps = list(model.parameters())
+        return cls([{"params": ps[:9]}, {"params": ps[9:], "weight_decay": 0.0}], **hyper)
+
+    native, python = build(a), build(b)
+    python.native_step = False
+    gen = torch.Generator().manual_seed(4)
+    for it in range(10):
+        grads = [(torch.randn(p.shape, generator=gen) * 1e-3).to(p.dtype).to(hip_device) for p in a.parameters()]
+        if it == 3:
+            for opt in (native, python):
+                opt.param_groups[0]["lr"] *= 0.5
+        if it == 5:
+            for opt in (native, python):
+                opt.load_state_dict(opt.state_dict())
+        if it == 7:
+            for opt, model in ((native, a), (python, b)):
+                st = opt.state[model.ps[4]]
+                st["exp_avg"] = st["exp_avg"].clone().mul_(0.5)
+        for model in (a, b):
+            for i, (p, g) in enumerate(zip(model.parameters(), grads)):
+                late = i == 2 and it < 4            # first gradient on the fifth step
+                skipped = i == 6 and it % 3 == 1    # no gradient now and then
+                p.grad = None if (late or skipped or it == 8) else g.clone()
+        native.step()
+        python.step()
+    for i, (pa, pb) in enumerate(zip(a.parameters(), b.parameters())):
+        G.assert_bits_equal(pa, pb, f"{case} param {i}")
+        assert list(native.state[pa].keys()) == list(python.state[pb].keys())
+        for key, val in native.state[pa].items():
+            if torch.is_tensor(val) and val.is_cuda and val.is_floating_point():
+                G.assert_bits_equal(val, python.state[pb][key], f"{case} {key} {i}")
+    for ga, gb in zip(native.param_groups, python.param_groups):
+        if "step" in ga:
+            assert int(ga["step"]) == int(gb["step"]) == 10
+    assert not torch.equal(a.ps[0], ManySmall(hip_device).ps[0]), "nothing was stepped"
+
+
+def test_step_hooks_and_profiler_ranges_survive_the_fast_step(hip_device):
+    """step() skips torch's wrapper only when it has nothing to do: hooks registered later fire,
+    with the arguments torch's wrapper would hand them, and a profiler sees the step's range."""
+    model, params = make(torch.bfloat16, hip_device)
+    opt = optimi_amd.AdamW(params, lr=1e-3)
+    loss_step(model, torch.bfloat16, hip_device, torch.Generator().manual_seed(0))
+    opt.step()
+    seen = []
+    pre = opt.register_step_pre_hook(lambda o, args, kwargs: seen.append(("pre", o is opt)))
+    post = opt.register_step_post_hook(lambda o, args, kwargs: seen.append(("post", kwargs.get("param"))))
+    opt.step()
+    assert seen == [("pre", True), ("post", None)]
+    pre.remove()
+    post.remove()
+    opt.step()
+    assert len(seen) == 2
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CPU]) as prof:
+        opt.step()
+    assert any("Optimizer.step#AdamW.step" in e.name for e in prof.events())
+    import warnings
+
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")  # the scheduler warns about step order if its wrapper did not see the step
+        sched = torch.optim.lr_scheduler.LambdaLR(opt, lambda e: 0.5)
+        opt.step()
+        sched.step()
+    assert opt.param_groups[0]["lr"] == 5e-4
