@@ -64,6 +64,20 @@ __device__ __forceinline__ void store16(void* base, int64_t byte_off, u32x4 v) {
   __builtin_nontemporal_store(v, (OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
 }
 
+// The store of a full tile: a buffer store with the sc0 sc1 cache policy, i.e. written through
+// to memory instead of left dirty in L2 (or marked for early eviction, as `nt` does).  With nine
+// streams per wave this is worth about 3 % of HBM bandwidth on MI355X: dirty lines evicted later
+// reach the DRAM out of step with the reads.  The clang builtin for global stores cannot
+// express the policy, the buffer builtin can, and unlike inline assembly it is tracked by the
+// compiler's wait-count insertion.  `tile` (wave-uniform) points at the workgroup's tile of
+// one array, `lane_off` is the lane's byte offset in it.
+constexpr int kStorePolicy = 1 | 16;  // aux bits of the buffer instructions on gfx94x/gfx950: 1 sc0, 2 nt, 16 sc1
+__device__ __forceinline__ void store16_tile(void* tile, uint32_t lane_off, u32x4 v) {
+  // dword 3 = 0x00020000: raw buffer, 32-bit data format; stride 0; bounds = the tile
+  __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(tile, 0, (uint32_t)(kThreads * kUnroll * 16), 0x00020000);
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_off, 0, kStorePolicy);
+}
+
 // Element math runs on pairs of neighbouring elements (f32x2): one v_cvt_pk_bf16_f32 then
 // rounds two values.  With packed fp32 ops disabled the pair arithmetic is two scalar ops.
 __device__ __forceinline__ f32x2 splat(float x) { return f32x2{x, x}; }
@@ -507,9 +521,11 @@ __device__ __forceinline__ double block_sum(double v, double* lds) {
 
 // Unpacks one 16-byte vector per loaded array, runs the element function on each pair and
 // writes the stored arrays back to element offset `off` of the tensor.
-template <class Op>
+// `TILE`: the workgroup owns a full tile starting at element `tile_base` (wave-uniform) and
+// stores through store16_tile; otherwise element `off` onwards is stored with plain stores.
+template <class Op, bool TILE = false>
 __device__ __forceinline__ void compute_store(const TensorEntry& e, int64_t off, const u32x4* raw,
-                                              const typename Op::Scalars& s, float& acc) {
+                                              const typename Op::Scalars& s, float& acc, int64_t tile_base = 0) {
   using DT = typename Op::DT;
   constexpr int P = DT::kPairs;
   constexpr int A = Op::kArrays;
@@ -534,7 +550,13 @@ __device__ __forceinline__ void compute_store(const TensorEntry& e, int64_t off,
   }
 #pragma unroll
   for (int a = 0; a < A; ++a)
-    if (Op::kStore & bit(a)) store16(e.ptr[a], off * DT::kElemBytes, DT::pack(f[a]));
+    if (Op::kStore & bit(a)) {
+      if (TILE)
+        store16_tile((void*)((uintptr_t)e.ptr[a] + (uintptr_t)(tile_base * DT::kElemBytes)),
+                     (uint32_t)((off - tile_base) * DT::kElemBytes), DT::pack(f[a]));
+      else
+        store16(e.ptr[a], off * DT::kElemBytes, DT::pack(f[a]));
+    }
 }
 
 template <class Op>
@@ -588,7 +610,7 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
     for (int u = 0; u < kUnroll; ++u) load_vec<Op>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u]);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
-      compute_store<Op>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u], s, acc);
+      compute_store<Op, true>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u], s, acc, base);
   } else if (e.vec_ok) {
     // end of a tensor: whole vectors while they fit, then the few leftover elements
     const int64_t end = e.numel;
@@ -868,23 +890,28 @@ int note_launch(optimi_group* g, hipStream_t stream) {
   return 0;
 }
 
-// Occupancy throttle.  HBM serves this read-modify-write mix best when a CU keeps only about
-// kStreamBudget 16-byte-per-lane vector streams (loads plus stores, counted per wavefront) in
-// flight; more resident wavefronts lower the achieved bandwidth.  The cap is imposed with a
-// dynamic-LDS request that no kernel touches: a CU has 160 KiB of LDS, so asking for L bytes
-// leaves room for floor(160 KiB / L) workgroups.  OPTIMI_HIP_STREAM_BUDGET overrides the budget
-// (0 = no throttle); it is read once.
-constexpr int kStreamBudgetDefault = 86;
+// Occupancy throttle.  HBM serves this read-modify-write mix best when a CU keeps only a
+// certain number of wavefronts resident - fewer the more 16-byte-per-lane streams (loads plus
+// stores) each wavefront carries; beyond it the achieved bandwidth drops by several per cent,
+// below it the CU cannot cover the latency.  The table is the measured optimum on MI355X with
+// the write-through tile stores (7B-parameter lists; 5 streams = StableAdamW pass 1, 6 = pass
+// 2, 7 = Lion / SGD, 9 = Adam with Kahan, 13 = Adan; entries in between are interpolated).
+// fp32 lists with 7 streams do best one wavefront above the 16-bit ones.  The cap is imposed
+// with a dynamic-LDS request that no kernel touches: a CU has 160 KiB of LDS, so asking for L
+// bytes leaves room for floor(160 KiB / L) workgroups.  OPTIMI_HIP_WAVES overrides the number
+// of wavefronts per CU for every kernel (0 = no throttle); it is read once.
 constexpr int kLdsPerCu = 160 * 1024;
+constexpr int kMaxStreams = 2 * kMaxArrays;
+constexpr int kBestWaves[kMaxStreams + 1] = {32, 32, 32, 32, 24, 17, 17, 12, 12, 11, 10, 9, 8, 8, 8};
 
-int stream_budget() {
+int forced_waves() {
 #ifdef OPTIMI_TUNING
-  if (const char* env = std::getenv("OPTIMI_HIP_STREAM_BUDGET")) return (int)std::strtol(env, nullptr, 10);
+  if (const char* env = std::getenv("OPTIMI_HIP_WAVES")) return (int)std::strtol(env, nullptr, 10);
+  return -1;
 #endif
   static const int value = [] {
-    long v = kStreamBudgetDefault;
-    if (const char* env = std::getenv("OPTIMI_HIP_STREAM_BUDGET")) v = std::strtol(env, nullptr, 10);
-    return (int)(v < 0 ? 0 : v);
+    const char* env = std::getenv("OPTIMI_HIP_WAVES");
+    return env ? (int)std::strtol(env, nullptr, 10) : -1;
   }();
   return value;
 }
@@ -893,10 +920,12 @@ constexpr int popcount(uint32_t x) { return x ? (int)(x & 1u) + popcount(x >> 1)
 
 template <class Op>
 unsigned throttle_lds() {
-  const int budget = stream_budget();
-  if (budget <= 0) return 0;
   constexpr int streams = (popcount(Op::kLoad) + popcount(Op::kStore)) * kUnroll;
-  int waves = (2 * budget + streams) / (2 * streams);  // round(budget / streams)
+  constexpr bool f32 = std::is_same<typename Op::DT, F32>::value;
+  int waves = kBestWaves[streams < kMaxStreams ? streams : kMaxStreams] + ((f32 && streams == 7) ? 1 : 0);
+  const int forced = forced_waves();
+  if (forced == 0) return 0;
+  if (forced > 0) waves = forced;
   int wgs = waves / (kThreads / 64);
   if (wgs < 1) wgs = 1;
   // midway between "wgs fit" and "wgs + 1 fit", so allocation granularity cannot tip it
