@@ -1,71 +1,69 @@
-"""Gradient release: run the optimizer step for a parameter as soon as its gradient has been
-accumulated, then free the gradient (optimi/gradientrelease.py:13-61)."""
+"""Gradient release: each parameter is stepped the moment autograd has finished accumulating
+its gradient, and the gradient is freed right after, so a full set of gradients never exists
+at once.  Same entry points and error behaviour as optimi/gradientrelease.py:13-61; the hook
+itself is native (see ``OptimiOptimizer._native_hook``)."""
 
 from __future__ import annotations
 
-from warnings import warn
+import warnings
 
-from torch import Tensor
-from torch.nn import Module
+import torch
 
 from .optimizers import OptimiOptimizer
 
 __all__ = ["prepare_for_gradient_release", "remove_gradient_release"]
 
+_HOOKS_ATTR = "_gradient_release_hooks"
+_OPTIMIZER_ATTR = "_gradient_release_optimizer"
 
-def _gradient_release_hook(param: Tensor, optimizer: OptimiOptimizer):
-    """What every registered hook does: ``step(param=param)`` then ``zero_grad(param=param)``
-    (optimi/gradientrelease.py:13-15).  The hooks registered below are the native form of this
-    function (state and group lookup, scalar prologue, launch or parking, freeing the gradient,
-    without a Python frame per parameter); this Python form gives the same results."""
+
+def _gradient_release_hook(param: torch.Tensor, optimizer: OptimiOptimizer):
+    """Python form of the hook, kept as the definition of what the native hook must do (the
+    tests run the two side by side): step this parameter, then drop its gradient
+    (optimi/gradientrelease.py:13-15)."""
     optimizer._release(param)
 
 
-def prepare_for_gradient_release(model: Module, optimizer: OptimiOptimizer, ignore_existing_hooks: bool = False):
-    """Register post_accumulate_grad_hooks on parameters for the gradient release optimization step.
+def _has_foreign_hooks(param: torch.Tensor) -> bool:
+    hooks = param._post_accumulate_grad_hooks
+    return hooks is not None and len(hooks) > 0
 
-    Args:
-        model: Model to register post_accumulate_grad_hooks. Only registers on parameters with
-            `requires_grad=True`.
-        optimizer: Optimizer providing the fused optimizer step during the backward pass. Requires
-            optimizer to be initialized with `gradient_release=True`
-        ignore_existing_hooks: If True, ignores existing post_accumulate_grad_hooks on parameters
-            and registers gradient release hooks (default: False)
+
+def prepare_for_gradient_release(model: torch.nn.Module, optimizer: OptimiOptimizer, ignore_existing_hooks: bool = False):
+    """Attach the gradient-release step to every trainable parameter of ``model``.
+
+    ``optimizer`` must be an optimi_amd optimizer constructed with ``gradient_release=True``
+    (``TypeError`` / ``ValueError`` otherwise).  A parameter that already carries a
+    post-accumulate-grad hook is an error - nothing is registered then - unless
+    ``ignore_existing_hooks`` is set.  Undo with ``remove_gradient_release``.
     """
     if not isinstance(optimizer, OptimiOptimizer):
         raise TypeError("`optimizer` must be an instance of `OptimiOptimizer`")
     if not optimizer.defaults["gradient_release"]:
         raise ValueError("`optimizer` must be initialized with `gradient_release=True`")
 
-    hook = optimizer._native_hook()
-    registered = []
-    for p in model.parameters():
-        if not p.requires_grad:
-            continue
-        existing = p._post_accumulate_grad_hooks
-        if existing is not None and len(existing) > 0 and not ignore_existing_hooks:
-            for handle in registered:
-                handle.remove()
-            raise ValueError(
-                "Model already has post_accumulate_grad_hooks. If this is expected, rerun with `ignore_existing_hooks=True`."
-            )
-        registered.append(p.register_post_accumulate_grad_hook(hook))
-    model._gradient_release_hooks = registered
-    # the hooks refer to the optimizer weakly; the model keeps it alive, as the reference's hooks do
-    model._gradient_release_optimizer = optimizer
+    trainable = [p for p in model.parameters() if p.requires_grad]
+    if not ignore_existing_hooks and any(_has_foreign_hooks(p) for p in trainable):
+        raise ValueError(
+            "Model already has post_accumulate_grad_hooks. If this is expected, rerun with `ignore_existing_hooks=True`."
+        )
+
+    hook = optimizer._native_hook()  # one callable for all parameters
+    setattr(model, _HOOKS_ATTR, [p.register_post_accumulate_grad_hook(hook) for p in trainable])
+    # the native hook refers to its optimizer weakly; the model keeps the optimizer alive for as
+    # long as the hooks are in place, which is what the reference's closures do implicitly
+    setattr(model, _OPTIMIZER_ATTR, optimizer)
 
 
-def remove_gradient_release(model: Module):
-    """Removes post_accumulate_grad_hooks created by `prepare_for_gradient_release`.
-
-    Args:
-        model: Model to remove gradient release post_accumulate_grad_hooks from.
-    """
-    if not hasattr(model, "_gradient_release_hooks"):
-        warn("`model` does not have any gradient release post_accumulate_grad_hooks to remove.")
+def remove_gradient_release(model: torch.nn.Module):
+    """Detach the hooks ``prepare_for_gradient_release`` put on ``model``'s parameters; warns if
+    there are none."""
+    handles = getattr(model, _HOOKS_ATTR, None)
+    if handles is None:
+        warnings.warn("`model` does not have any gradient release post_accumulate_grad_hooks to remove.")
         return
-    for handle in model._gradient_release_hooks:
+    for handle in handles:
         handle.remove()
-    del model._gradient_release_hooks
-    if hasattr(model, "_gradient_release_optimizer"):
-        del model._gradient_release_optimizer
+    delattr(model, _HOOKS_ATTR)
+    if hasattr(model, _OPTIMIZER_ATTR):
+        delattr(model, _OPTIMIZER_ATTR)
