@@ -73,6 +73,11 @@ def workloads():
 MEASURED_TRAFFIC_BYTES = {
     # profiles/adamw_bf16_kahan_llama7b_hbm_traffic.txt: 67.44 GB read + 53.90 GB written
     "adamw_bf16_kahan_llama7b": 1.2134e11,
+    # profiles/lion_stableadamw_adan_adamw1b_hbm_traffic.txt
+    "lion_bf16_kahan_llama7b": 9.439e10,
+    "stableadamw_bf16_kahan_llama7b": 1.4887e11,
+    "adan_bf16_kahan_llama7b": 1.7524e11,
+    "adamw_bf16_kahan_declr_llama1b": 2.170e10,
 }
 
 
