@@ -555,12 +555,19 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
   }
 
   void flush() {
-    std::lock_guard<std::recursive_mutex> lock(mutex_);
-    if (batch_.empty()) return;
+    // The parked steps leave the queue under its lock and are launched, and their tensors let
+    // go, outside it: dropping the last reference to a tensor that Python knows takes the GIL,
+    // and a hook that holds the GIL may be waiting for the queue's lock at that moment.
     std::vector<StepCall> batch;
-    batch.swap(batch_);  // the queue is empty again whatever happens below
-    seen_.clear();
-    total_ = 0;
+    hipStream_t stream = nullptr;
+    {
+      std::lock_guard<std::recursive_mutex> lock(mutex_);
+      if (batch_.empty()) return;
+      batch.swap(batch_);
+      stream = stream_;
+      seen_.clear();
+      total_ = 0;
+    }
     const StepCall& c0 = batch[0];
     const int n = (int)batch.size(), nt = kTensorsOf[c0.kind];
     const int dtype = dtype_code(c0.param());
@@ -573,9 +580,10 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
         if (batch[(size_t)i].t[a].has_value()) ptr[a][(size_t)i] = batch[(size_t)i].t[a]->data_ptr();
     }
     c10::hip::HIPGuardMasqueradingAsCUDA guard(c0.param().device());
+    std::lock_guard<std::mutex> launching(launch_mutex_);  // the workspaces serve one launch at a time
     std::unique_ptr<Group>& slot = groups_[c0.param().device().index()];  // a workspace lives on one device
     if (!slot) slot = std::make_unique<Group>();  // made on first use: a queue may exist before any device work
-    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtype, c0.s, c0.flags, stream_);
+    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtype, c0.s, c0.flags, stream);
   }
 
  private:
@@ -601,6 +609,7 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
 
   int64_t max_numel_, max_tensors_, max_total_;
   std::recursive_mutex mutex_;
+  std::mutex launch_mutex_;
   int scheduled_task_ = -1;  // the backward pass that already carries the flush callback
   std::unordered_map<int, std::unique_ptr<Group>> groups_;
   std::vector<StepCall> batch_;
