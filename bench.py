@@ -320,7 +320,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
                      "bytes_per_param": bytes_per_param, "kernel_ms": mean_kernel_ms,
-                     "kernel_ms_min": min(kernel_ms), "kernel_ms_max": max(kernel_ms)},
+                     "kernel_ms_min": min(kernel_ms), "kernel_ms_max": max(kernel_ms),
+                     "kernel_ms_p50": sorted(kernel_ms)[len(kernel_ms) // 2],
+                     "kernel_ms_p90": sorted(kernel_ms)[min(len(kernel_ms) - 1, (len(kernel_ms) * 9) // 10)]},
         "cpu_baseline": None,
     }
     del opt, params, grad_sets
