@@ -28,13 +28,14 @@ _LOW_PRECISION = (torch.float16, torch.bfloat16)
 
 
 def _require_hip_backend(triton, foreach, gradient_release):
-    if foreach:
-        if gradient_release:
-            raise ValueError(f"Gradient release {gradient_release=} and foreach {foreach=} cannot be used together")
-        raise ValueError("optimi_amd has no foreach backend; use triton=True (served by the HIP kernels)")
-    if not triton:
+    """Both of the reference's accelerated selectors, ``triton=True`` and the deprecated
+    ``foreach=True``, are served by the HIP kernels; the PyTorch for-loop path (both False) does
+    not exist here.  foreach with gradient release is an error, as in optimi/adam.py:281-282."""
+    if foreach and gradient_release:
+        raise ValueError(f"Gradient release {gradient_release=} and foreach {foreach=} cannot be used together")
+    if not triton and not foreach:
         raise ValueError(
-            "optimi_amd implements only the fused HIP backend, selected with triton=True; "
+            "optimi_amd implements only the fused HIP backend, selected with triton=True (or foreach=True); "
             "the PyTorch for-loop path is not part of this package"
         )
 

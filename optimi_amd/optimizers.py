@@ -72,7 +72,13 @@ class OptimiOptimizer(Optimizer):
         if defaults["max_lr"] is not None and not 0.0 <= defaults["max_lr"]:
             raise ValueError(f"Invalid maximum learning rate: max_lr={defaults['max_lr']}")
         if defaults["foreach"]:
-            raise ValueError("optimi_amd has no foreach backend (the reference deprecates it); leave foreach unset")
+            # the reference deprecates foreach in favour of its fused backend (optimi/optimizer.py:33-38);
+            # here the flag selects the same HIP kernels as triton=True
+            warn(
+                "Parameter `foreach` is deprecated; optimi_amd serves foreach=True with the fused HIP kernels, as it does "
+                "triton=True. Set `foreach=False` or leave it unset to silence this warning.",
+                category=DeprecationWarning,
+            )
         if defaults["triton"] is False:
             raise ValueError("optimi_amd implements only the fused HIP backend; leave triton unset or pass triton=True")
 
@@ -94,6 +100,9 @@ class OptimiOptimizer(Optimizer):
         self._release_hook = None
 
         if self.defaults["gradient_release"]:
+            if self.defaults["foreach"]:  # optimi/optimizer.py:65-68
+                warn("Gradient release (gradient_release=True) and foreach (foreach=True) cannot be used together. "
+                     "Disabling foreach.", category=UserWarning)
             self.defaults["foreach"] = False
             for group in self.param_groups:
                 group["foreach"] = False
@@ -384,7 +393,7 @@ class Adam(OptimiOptimizer):
         kahan_sum: Enables Kahan summation for more accurate parameter updates when training in low
             precision (bfloat16). If unspecified, automatically applies for low precision
             parameters (default: None)
-        foreach: Not available in this package; must stay unset (default: None)
+        foreach: Deprecated. True selects the fused HIP kernels, like `triton=True` (default: None)
         triton: Selects the fused backend, here the HIP kernels. Unset or True (default: None)
         gradient_release: Fuses optimizer step and zero_grad as part of the parameter's backward
             pass. Requires model hooks created with `prepare_for_gradient_release`. Incompatible

@@ -420,3 +420,26 @@ def test_step_hooks_and_profiler_ranges_survive_the_fast_step(hip_device):
         opt.step()
         sched.step()
     assert opt.param_groups[0]["lr"] == 5e-4
+
+
+def test_foreach_true_selects_the_hip_kernels(hip_device):
+    """The reference's other accelerated selector: deprecated, accepted, same kernels and results
+    as triton=True; with gradient release it is switched off with a warning, as in the reference."""
+    import warnings
+
+    a, b = ManySmall(hip_device), ManySmall(hip_device)
+    with pytest.warns(DeprecationWarning, match="foreach"):
+        via_foreach = optimi_amd.AdamW(a.parameters(), lr=1e-3, foreach=True)
+    via_triton = optimi_amd.AdamW(b.parameters(), lr=1e-3, triton=True)
+    for it in range(3):
+        for model, opt in ((a, via_foreach), (b, via_triton)):
+            model(1.0 + it).backward()
+            opt.step()
+            opt.zero_grad()
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        G.assert_bits_equal(pa, pb, "foreach=True vs triton=True")
+    assert via_foreach.param_groups[0]["foreach"] is True
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = optimi_amd.AdamW(a.parameters(), lr=1e-3, foreach=True, gradient_release=True)
+    assert opt.param_groups[0]["foreach"] is False

@@ -39,7 +39,7 @@ def test_constructor_validation(cls):
     if cls not in NO_EPS:
         with pytest.raises(ValueError, match="epsilon"):
             cls(params(), lr=1e-3, eps=-1e-8)
-    with pytest.raises(ValueError, match="foreach"):
+    with pytest.warns(DeprecationWarning, match="foreach"):  # deprecated as in the reference; served by the HIP kernels
         cls(params(), lr=1e-3, foreach=True)
     with pytest.raises(ValueError, match="HIP backend"):
         cls(params(), lr=1e-3, triton=False)
@@ -100,8 +100,9 @@ def test_functional_forms_refuse_other_backends():
     kw = dict(lr=1e-3, beta1=0.9, beta2=0.99, weight_decay=0.0, eps=1e-6, step=step)
     with pytest.raises(ValueError, match="only the fused HIP backend"):
         F.adamw([p], [g], [m], [v], **kw)
-    with pytest.raises(ValueError, match="no foreach backend"):
+    with pytest.raises(RuntimeError, match="HIP devices only"):  # foreach=True selects the HIP kernels too
         F.adamw([p], [g], [m], [v], foreach=True, **kw)
+    step.zero_()
     with pytest.raises(ValueError, match="cannot be used together"):
         F.adamw(p, g, m, v, foreach=True, gradient_release=True, **kw)
     assert int(step) == 0  # rejected before the counter moved
