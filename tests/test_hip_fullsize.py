@@ -1,4 +1,4 @@
-"""Parity at the sizes of the BASELINE configurations.
+"""Parity at the sizes of the benchmark configurations.
 
 * C2 – AdamW bf16 + Kahan, ``decouple_lr``, wd 1e-5, the whole Llama-1B-shaped list (147 tensors,
   1,204,881,408 params), 10 steps with fresh gradients: every tensor against the C emulator, bit-exact.

@@ -188,7 +188,7 @@ def test_gradient_release_with_accumulation(cfg, dtype, hip_device):
 
 
 def test_baseline_config_adamw_fp32_mlp(hip_device):
-    """BASELINE config 1: AdamW fp32, 2 x [W1 1024x4096, b1 4096, W2 4096x1024, b2 1024], 10 steps, seed 0."""
+    """The small fp32 benchmark configuration: AdamW fp32, 2 x [W1 1024x4096, b1 4096, W2 4096x1024, b2 1024], 10 steps, seed 0."""
     from hip_engine import HipRun
 
     shapes = [(1024, 4096), (4096,), (4096, 1024), (1024,)] * 2
