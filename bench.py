@@ -229,7 +229,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adamw_bf16_kahan_llama7b")
     ap.add_argument("--grad-sets", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
