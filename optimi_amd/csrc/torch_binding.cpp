@@ -465,7 +465,8 @@ void launch_list(Kind kind, optimi_group* g, int n, const std::vector<void*>* pt
   const char* what = "";
   switch (kind) {
     case ADAM:
-      rc = optimi_hip_adam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], flags, stream);
+      rc = optimi_hip_adam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype,
+          s[0], s[1], s[2], s[3], s[4], s[5], flags, stream);
       what = "optimi_hip_adam_multi";
       break;
     case LION:
@@ -473,11 +474,13 @@ void launch_list(Kind kind, optimi_group* g, int n, const std::vector<void*>* pt
       what = "optimi_hip_lion_multi";
       break;
     case STABLEADAMW:
-      rc = optimi_hip_stableadamw_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], flags, stream);
+      rc = optimi_hip_stableadamw_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype,
+          s[0], s[1], s[2], s[3], s[4], s[5], s[6], flags, stream);
       what = "optimi_hip_stableadamw_multi";
       break;
     case ADAN:
-      rc = optimi_hip_adan_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), arr(5), opt(6), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], flags, stream);
+      rc = optimi_hip_adan_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), arr(5), opt(6), numel, dtype,
+          s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], flags, stream);
       what = "optimi_hip_adan_multi";
       break;
     case SGD:
@@ -485,11 +488,13 @@ void launch_list(Kind kind, optimi_group* g, int n, const std::vector<void*>* pt
       what = "optimi_hip_sgd_multi";
       break;
     case RADAM:
-      rc = optimi_hip_radam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], flags, stream);
+      rc = optimi_hip_radam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype,
+          s[0], s[1], s[2], s[3], s[4], s[5], s[6], flags, stream);
       what = "optimi_hip_radam_multi";
       break;
     case RANGER:
-      rc = optimi_hip_ranger_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), opt(5), numel, dtype, s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], flags, stream);
+      rc = optimi_hip_ranger_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), opt(5), numel, dtype,
+          s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], flags, stream);
       what = "optimi_hip_ranger_multi";
       break;
   }
