@@ -194,6 +194,10 @@ def release_bench(args):
     opt = optimi_amd.AdamW(params, gradient_release=True, **kwargs)
     if args.no_coalesce:
         opt.gradient_release_coalesce = 0
+    if args.coalesce_numel is not None:
+        opt.gradient_release_coalesce = args.coalesce_numel
+    if args.coalesce_window is not None:
+        opt._QUEUE_MAX_ELEMENTS = args.coalesce_window
     optimi_amd.prepare_for_gradient_release(model, opt)
 
     def one_pass(i):
@@ -238,6 +242,10 @@ def main():
     ap.add_argument("--copy-probe-bytes", type=int, default=0,
                     help="also run the library's plain copy kernel over this many bytes (3 launches) before the "
                          "workload; a profiler run uses it to scale its byte counters against a known size")
+    ap.add_argument("--coalesce-numel", type=int, default=None,
+                    help="gradient-release workloads: park tensors of at most this many elements (default: the optimizer's)")
+    ap.add_argument("--coalesce-window", type=int, default=None,
+                    help="gradient-release workloads: launch when this many elements are parked (default: the optimizer's)")
     args = ap.parse_args()
 
     if args.gpus != 1:
