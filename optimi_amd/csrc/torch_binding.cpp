@@ -14,7 +14,9 @@
 #include <torch/csrc/autograd/python_variable.h>
 #include <torch/extension.h>
 
+#include <atomic>
 #include <cmath>
+#include <cstdio>
 #include <cstring>
 #include <memory>
 #include <mutex>
@@ -501,6 +503,21 @@ void launch_list(Kind kind, optimi_group* g, int n, const std::vector<void*>* pt
   check_status(rc, what);
 }
 
+// What the per-tensor entry points check before they launch, for a step that may be parked
+// instead.  Run before the step counter advances, so that a rejected step leaves no trace.
+void validate_call(const StepCall& c) {
+  static const char* const names[] = {"param", "grad", "state", "state", "state", "state", "state"};
+  const at::Tensor& p = c.param();
+  check_param(p);
+  (void)dtype_code(p);
+  for (int a = 1; a < kTensorsOf[c.kind]; ++a)
+    if (c.t[a].has_value()) check_like(p, *c.t[a], names[a]);
+}
+
+void check_hip(hipError_t err, const char* what) {
+  TORCH_CHECK(err == hipSuccess, "optimi_amd: ", what, " failed: ", hipGetErrorString(err));
+}
+
 // Parks the steps of small tensors and launches them together, as one list per run of steps
 // that share everything but their tensors (optimizer, dtype, device, stream, flags and every
 // scalar - which includes the step count through the debiased betas).  A tensor of a few
@@ -518,7 +535,12 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
   ReleaseQueue(int64_t max_numel, int64_t max_tensors, int64_t max_total)
       : max_numel_(max_numel), max_tensors_(max_tensors), max_total_(max_total) {}
   ~ReleaseQueue() {
-    // steps still parked are dropped, never launched from a destructor (the device may be gone)
+    // steps still parked are dropped, never launched from a destructor (the device may be gone);
+    // their step counters have advanced, so say so
+    if (!batch_.empty())
+      std::fprintf(stderr, "optimi_amd: a gradient-release queue was destroyed with %zu parked optimizer steps that "
+                           "were never launched (flush it, e.g. through optimizer.step() or state_dict(), first)\n",
+                   batch_.size());
   }
 
   bool wants(const StepCall& c) const {
@@ -528,6 +550,9 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
     std::lock_guard<std::recursive_mutex> lock(mutex_);
     return (int64_t)batch_.size();
   }
+  // list launches made so far, and the per-tensor steps they carried
+  int64_t launches() const { return launches_; }
+  int64_t launched_steps() const { return launched_steps_; }
 
   // Makes sure the running backward pass ends with a flush.
   void schedule() {
@@ -541,7 +566,7 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
           std::lock_guard<std::recursive_mutex> inner(q->mutex_);
           q->scheduled_task_ = -1;
         }
-        q->flush();
+        q->flush(/*end_of_backward=*/true);
       }
     });
     scheduled_task_ = task;
@@ -549,7 +574,6 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
 
   void add(StepCall&& c) {
     std::lock_guard<std::recursive_mutex> lock(mutex_);
-    validate(c);
     const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(c.param().device().index()).stream();
     if (!batch_.empty() && (!same_run(c, stream) || seen_.count(c.param().data_ptr()))) flush();
     if (batch_.empty()) stream_ = stream;
@@ -559,7 +583,14 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
     if ((int64_t)batch_.size() >= max_tensors_ || total_ >= max_total_) flush();
   }
 
-  void flush() {
+  // `end_of_backward`: called from the autograd engine's final callback.  The engine runs those
+  // under the streams that were current when backward() was called, after making them wait for
+  // the streams the gradients were accumulated on - so there the launch goes to the device's
+  // current stream, which is where the caller's next work (the next forward, step(),
+  // state_dict()) is ordered.  Everywhere else the launch goes to the stream the steps were
+  // parked on (the stream their gradients are ready on), and when that is not the current
+  // stream, the current stream is made to wait for the launch.
+  void flush(bool end_of_backward = false) {
     // The parked steps leave the queue under its lock and are launched, and their tensors let
     // go, outside it: dropping the last reference to a tensor that Python knows takes the GIL,
     // and a hook that holds the GIL may be waiting for the queue's lock at that moment.
@@ -588,19 +619,28 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
     std::lock_guard<std::mutex> launching(launch_mutex_);  // the workspaces serve one launch at a time
     std::unique_ptr<Group>& slot = groups_[c0.param().device().index()];  // a workspace lives on one device
     if (!slot) slot = std::make_unique<Group>();  // made on first use: a queue may exist before any device work
-    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtype, c0.s, c0.flags, stream);
+    const auto current_stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(c0.param().device().index());
+    const hipStream_t current = current_stream.stream();
+    const hipStream_t launch = end_of_backward ? current : stream;
+    if (launch != stream) {
+      // The parked gradients were allocated on the stream they were parked on and are let go as
+      // soon as this function returns: tell the caching allocator that another stream reads them.
+      for (const StepCall& c : batch) c.t[1]->record_stream(current_stream);
+    }
+    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtype, c0.s, c0.flags, launch);
+    ++launches_;
+    launched_steps_ += n;
+    if (launch != current) {
+      hipEvent_t done = nullptr;
+      check_hip(hipEventCreateWithFlags(&done, hipEventDisableTiming), "hipEventCreateWithFlags");
+      hipError_t err = hipEventRecord(done, launch);
+      if (err == hipSuccess) err = hipStreamWaitEvent(current, done, 0);
+      (void)hipEventDestroy(done);  // the runtime keeps a recorded event alive until it has completed
+      check_hip(err, "ordering the current stream after the gradient-release launch");
+    }
   }
 
  private:
-  // what the per-tensor entry points check before they launch
-  static void validate(const StepCall& c) {
-    static const char* const names[] = {"param", "grad", "state", "state", "state", "state", "state"};
-    const at::Tensor& p = c.param();
-    check_param(p);
-    (void)dtype_code(p);
-    for (int a = 1; a < kTensorsOf[c.kind]; ++a)
-      if (c.t[a].has_value()) check_like(p, *c.t[a], names[a]);
-  }
 
   bool same_run(const StepCall& c, hipStream_t stream) const {
     const StepCall& c0 = batch_[0];
@@ -621,6 +661,7 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
   std::unordered_set<void*> seen_;
   int64_t total_ = 0;
   hipStream_t stream_ = nullptr;
+  std::atomic<int64_t> launches_{0}, launched_steps_{0};
 };
 
 // Parks the step when there is a queue, a backward pass is running and the tensor is small
@@ -698,45 +739,55 @@ Hyper ranger_hyper(int64_t t, bool lookahead, double lr, double beta1, double be
                   rect >= 0 ? rect : 0.0, alpha}};
 }
 
-StepCall make_call(Kind kind, const Hyper& h, std::initializer_list<std::optional<at::Tensor>> tensors) {
+// The tensors of one step, validated; the scalars follow through set_hyper once the step
+// counter has been advanced - nothing is mutated for a step that is rejected here.
+StepCall make_call(Kind kind, std::initializer_list<std::optional<at::Tensor>> tensors) {
   StepCall c;
   c.kind = kind;
-  c.flags = h.flags;
-  std::memcpy(c.s, h.s, sizeof(c.s));
   int a = 0;
   for (const auto& t : tensors) c.t[a++] = t;
+  validate_call(c);
   return c;
+}
+
+StepCall&& set_hyper(StepCall&& c, const Hyper& h) {
+  c.flags = h.flags;
+  std::memcpy(c.s, h.s, sizeof(c.s));
+  return std::move(c);
 }
 
 bool adam_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
                   const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
                   double weight_decay, double eps, bool decouple_wd, bool decouple_lr, std::optional<double> max_lr,
                   bool kahan_sum, bool update, ReleaseQueue* queue) {
+  StepCall c = make_call(ADAM, {p, grad_like(p, g), m, v, real_kahan(p, k)});
   const Hyper h = adam_hyper(tick(step), lr, beta1, beta2, weight_decay, eps, decouple_wd, decouple_lr, max_lr, kahan_sum, update);
-  return submit(make_call(ADAM, h, {p, grad_like(p, g), m, v, real_kahan(p, k)}), queue);
+  return submit(set_hyper(std::move(c), h), queue);
 }
 
 bool lion_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const std::optional<at::Tensor>& k,
                   double lr, double beta1, double beta2, double weight_decay, bool decouple_lr,
                   std::optional<double> max_lr, bool kahan_sum, bool update, ReleaseQueue* queue) {
   const Hyper h = lion_hyper(lr, beta1, beta2, weight_decay, decouple_lr, max_lr, kahan_sum, update);
-  return submit(make_call(LION, h, {p, grad_like(p, g), m, real_kahan(p, k)}), queue);
+  return submit(set_hyper(make_call(LION, {p, grad_like(p, g), m, real_kahan(p, k)}), h), queue);
 }
 
 bool stableadamw_release(Group& group, const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
                          const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1, double beta2,
                          double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum,
                          bool update, ReleaseQueue* queue) {
+  StepCall c = make_call(STABLEADAMW, {p, grad_like(p, g), m, v, real_kahan(p, k)});
   const Hyper h = stableadamw_hyper(tick(step), lr, beta1, beta2, weight_decay, eps, decouple_lr, max_lr, kahan_sum, update);
-  return submit(make_call(STABLEADAMW, h, {p, grad_like(p, g), m, v, real_kahan(p, k)}), queue, &group);
+  return submit(set_hyper(std::move(c), h), queue, &group);
 }
 
 bool adan_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& df, const at::Tensor& n,
                   const at::Tensor& pg, const std::optional<at::Tensor>& k, const at::Tensor& step, double lr, double beta1,
                   double beta2, double beta3, double weight_decay, double eps, bool decouple_lr, std::optional<double> max_lr,
                   bool adam_wd, bool kahan_sum, bool update, ReleaseQueue* queue) {
+  StepCall c = make_call(ADAN, {p, grad_like(p, g), m, df, n, pg, real_kahan(p, k)});
   const Hyper h = adan_hyper(tick(step), lr, beta1, beta2, beta3, weight_decay, eps, decouple_lr, max_lr, adam_wd, kahan_sum, update);
-  return submit(make_call(ADAN, h, {p, grad_like(p, g), m, df, n, pg, real_kahan(p, k)}), queue);
+  return submit(set_hyper(std::move(c), h), queue);
 }
 
 bool sgd_release(const at::Tensor& p, const at::Tensor& g, const std::optional<at::Tensor>& m,
@@ -744,7 +795,7 @@ bool sgd_release(const at::Tensor& p, const at::Tensor& g, const std::optional<a
                  bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update,
                  ReleaseQueue* queue) {
   const Hyper h = sgd_hyper(lr, momentum, weight_decay, dampening, decouple_wd, decouple_lr, max_lr, kahan_sum, update);
-  return submit(make_call(SGD, h, {p, grad_like(p, g), momentum != 0 ? real_kahan(p, m) : std::nullopt, real_kahan(p, k)}), queue);
+  return submit(set_hyper(make_call(SGD, {p, grad_like(p, g), momentum != 0 ? real_kahan(p, m) : std::nullopt, real_kahan(p, k)}), h), queue);
 }
 
 bool ranger_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& m, const at::Tensor& v,
@@ -753,10 +804,11 @@ bool ranger_release(const at::Tensor& p, const at::Tensor& g, const at::Tensor& 
                     bool decouple_wd, bool decouple_lr, std::optional<double> max_lr, bool kahan_sum, bool update,
                     ReleaseQueue* queue) {
   // la = None makes this RAdam; with la it is Ranger
+  StepCall c = la.has_value() ? make_call(RANGER, {p, grad_like(p, g), m, v, *la, real_kahan(p, k)})
+                              : make_call(RADAM, {p, grad_like(p, g), m, v, real_kahan(p, k)});
   const Hyper h = ranger_hyper(tick(step), la.has_value(), lr, beta1, beta2, weight_decay, eps, sync_every, alpha, decouple_wd,
                                decouple_lr, max_lr, kahan_sum, update);
-  if (la.has_value()) return submit(make_call(RANGER, h, {p, grad_like(p, g), m, v, *la, real_kahan(p, k)}), queue);
-  return submit(make_call(RADAM, h, {p, grad_like(p, g), m, v, real_kahan(p, k)}), queue);
+  return submit(set_hyper(std::move(c), h), queue);
 }
 
 
@@ -813,8 +865,9 @@ class ReleaseHookCore {
     at::NoGradGuard no_grad;
     const bool update = !truthy(py::reinterpret_steal<py::object>(attr(optimizer.ptr(), k_.accumulation)).ptr());
     PyObject* grp = e->group.ptr();
-    const Hyper h = read_hyper(grp, has_step_ ? tick(e->step) : 0, update);
-    submit(pack(*e, h, p, grad_like(p, g), num_or_zero(grp)), queue_.get(), e->workspace);
+    StepCall c = pack(*e, Hyper{}, p, grad_like(p, g), num_or_zero(grp));
+    validate_call(c);  // before the counter moves: a rejected step leaves the state as it was
+    submit(set_hyper(std::move(c), read_hyper(grp, has_step_ ? tick(e->step) : 0, update)), queue_.get(), e->workspace);
     p.mutable_grad().reset();  // param.grad = None
   }
 
@@ -838,6 +891,7 @@ class ReleaseHookCore {
       Entry* e;
     };
     std::vector<Item> items;
+    const double momentum = num_or_zero(grp);
     const Py_ssize_t n_params = PyList_GET_SIZE(plist);
     items.reserve((size_t)n_params);
     for (Py_ssize_t i = 0; i < n_params; ++i) {
@@ -849,8 +903,9 @@ class ReleaseHookCore {
       TORCH_CHECK(!g.is_sparse(), "optimi_amd does not support sparse gradients");
       Entry* e = find(p);
       if (!e || !valid(*e, false)) e = refresh(optimizer, k_.group_entry, py::handle(obj), p, false, group);
-      check_param(p);
-      items.push_back({p, grad_like(p, g), e});
+      at::Tensor g_like = grad_like(p, g);
+      validate_call(pack(*e, Hyper{}, p, g_like, momentum));  // everything that can reject the step, before the counter moves
+      items.push_back({p, std::move(g_like), e});
     }
 
     // the group's counter advances even when nothing has a gradient, as in the reference
@@ -862,7 +917,6 @@ class ReleaseHookCore {
     }
     if (items.empty()) return true;
     const Hyper h = read_hyper(grp, t, true);
-    const double momentum = num_or_zero(grp);
 
     // pass 2: one launch per (device, dtype), in order of first appearance
     const int nt = kTensorsOf[kind_];
@@ -877,8 +931,6 @@ class ReleaseHookCore {
         if (done[i] || p.scalar_type() != p0.scalar_type() || p.device() != p0.device()) continue;
         done[i] = 1;
         const StepCall c = pack(*items[i].e, h, p, items[i].g, momentum);
-        for (int a = 1; a < nt; ++a)
-          if (c.t[a].has_value()) check_like(p, *c.t[a], a == 1 ? "grad" : "state");
         for (int a = 0; a < nt; ++a) ptr[a].push_back(c.t[a].has_value() ? c.t[a]->data_ptr() : nullptr);
         numel.push_back(p.numel());
       }
@@ -1134,8 +1186,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.attr("KIND_RANGER") = (int)RANGER;
   py::class_<ReleaseQueue, std::shared_ptr<ReleaseQueue>>(mod, "ReleaseQueue")
       .def(py::init<int64_t, int64_t, int64_t>(), py::arg("max_numel"), py::arg("max_tensors"), py::arg("max_total"))
-      .def("flush", &ReleaseQueue::flush)
-      .def("pending", &ReleaseQueue::pending);
+      .def("flush", [](ReleaseQueue& q) { q.flush(); })
+      .def("pending", &ReleaseQueue::pending)
+      .def("launches", &ReleaseQueue::launches)
+      .def("launched_steps", &ReleaseQueue::launched_steps);
   mod.def("adam_multi", &adam_multi);
   mod.def("lion_multi", &lion_multi);
   mod.def("stableadamw_multi", &stableadamw_multi);

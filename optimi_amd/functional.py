@@ -82,6 +82,40 @@ def _grads_like(params, grads):
     return out
 
 
+def _check_state(param: Tensor, state: Tensor, name: str):
+    if state.device != param.device or state.dtype != param.dtype or state.numel() != param.numel() \
+            or state.stride() != param.stride():
+        raise RuntimeError(f"optimi_amd: {name} must have the parameter's device, dtype, size and strides "
+                           f"(got {state.dtype} {tuple(state.shape)} on {state.device})")
+
+
+def _validated(params, grads, states, kahan_comps, optional=()):
+    """The two calling forms (lists, or bare tensors in gradient-release mode) as lists, with every
+    check that can reject the call done here - before the step counter moves or a kernel runs.
+    ``states`` are the per-parameter state columns; a column named in ``optional`` may hold None or
+    one-element placeholders."""
+    n = 1 if isinstance(params, Tensor) else len(params)
+    if kahan_comps is None:
+        kahan_comps = [None] * n
+    cols = _as_lists(params, grads, *states, kahan_comps)
+    params = cols[0]
+    for c in cols[1:]:
+        if len(c) != len(params):
+            raise ValueError(f"optimi_amd: got {len(params)} parameters but a list of {len(c)} gradients or states")
+    for p in params:
+        backend.check_supported(p)
+    cols[1] = _grads_like(params, cols[1])
+    for j, col in enumerate(cols[2:-1]):
+        for p, st in zip(params, col):
+            if j in optional and _real_kahan(p, st) is None:
+                continue
+            _check_state(p, st, "a state tensor")
+    for p, k in zip(params, cols[-1]):
+        if _real_kahan(p, k) is not None:
+            _check_state(p, k, "kahan_comp")
+    return cols
+
+
 # --------------------------------------------------------------------------------------
 # Adam / AdamW
 # --------------------------------------------------------------------------------------
@@ -116,6 +150,7 @@ def adam(
     """
     _require_hip_backend(triton, foreach, gradient_release)
     ext = backend.ext()
+    params, grads, exp_avgs, exp_avg_sqs, kahan_comps = _validated(params, grads, (exp_avgs, exp_avg_sqs), kahan_comps)
 
     t = _tick(step)
     beta1_hat = debias_beta(beta1, t)
@@ -129,14 +164,8 @@ def adam(
                    DECOUPLE_WD=decouple_wd or decouple_lr)
     scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps, flags)
 
-    if kahan_comps is None:
-        kahan_comps = [None] * (1 if isinstance(params, Tensor) else len(params))
-    params, grads, exp_avgs, exp_avg_sqs, kahan_comps = _as_lists(params, grads, exp_avgs, exp_avg_sqs, kahan_comps)
-    grads = _grads_like(params, grads)
-
     if gradient_release:
         for p, g, m, v, k in zip(params, grads, exp_avgs, exp_avg_sqs, kahan_comps):
-            backend.check_supported(p)
             ext.adam_single(p, g, m, v, _real_kahan(p, k), *scalars)
         return
     for (device, dtype), idxs in _buckets(params).items():
@@ -200,6 +229,7 @@ def lion(
     """Functional API to apply a Lion optimization step (optimi/lion.py:187-266)."""
     _require_hip_backend(triton, foreach, gradient_release)
     ext = backend.ext()
+    params, grads, exp_avgs, kahan_comps = _validated(params, grads, (exp_avgs,), kahan_comps)
 
     if weight_decay != 0:
         if decouple_lr:
@@ -209,14 +239,8 @@ def lion(
     flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation)
     scalars = (lr, 1 - beta1, 1 - beta2, weight_decay, flags)
 
-    if kahan_comps is None:
-        kahan_comps = [None] * (1 if isinstance(params, Tensor) else len(params))
-    params, grads, exp_avgs, kahan_comps = _as_lists(params, grads, exp_avgs, kahan_comps)
-    grads = _grads_like(params, grads)
-
     if gradient_release:
         for p, g, m, k in zip(params, grads, exp_avgs, kahan_comps):
-            backend.check_supported(p)
             ext.lion_single(p, g, m, _real_kahan(p, k), *scalars)
         return
     for (device, dtype), idxs in _buckets(params).items():
@@ -261,6 +285,9 @@ def stableadamw(
     """
     _require_hip_backend(triton, foreach, gradient_release)
     ext = backend.ext()
+    params, grads, exp_avgs, exp_avg_sqs, kahan_comps = _validated(params, grads, (exp_avgs, exp_avg_sqs), kahan_comps)
+    if decouple_lr and weight_decay != 0 and not (max_lr is not None and max_lr > 0):
+        raise ValueError(f"optimi_amd: decouple_lr needs a positive max_lr, got {max_lr=}")
 
     t = _tick(step)
     beta1_hat = debias_beta(beta1, t)
@@ -269,14 +296,8 @@ def stableadamw(
     scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps,
                float(max_lr) if (decouple_lr and max_lr is not None) else 0.0, flags)
 
-    if kahan_comps is None:
-        kahan_comps = [None] * (1 if isinstance(params, Tensor) else len(params))
-    params, grads, exp_avgs, exp_avg_sqs, kahan_comps = _as_lists(params, grads, exp_avgs, exp_avg_sqs, kahan_comps)
-    grads = _grads_like(params, grads)
-
     if gradient_release:
         for p, g, m, v, k in zip(params, grads, exp_avgs, exp_avg_sqs, kahan_comps):
-            backend.check_supported(p)
             grp = _workspace(_groups, p.device, p.dtype, "stableadamw_single")
             ext.stableadamw_single(grp, p, g, m, v, _real_kahan(p, k), *scalars)
         return
@@ -318,6 +339,8 @@ def adan(
     """Functional API to apply an Adan optimization step (optimi/adan.py:236-350)."""
     _require_hip_backend(triton, foreach, gradient_release)
     ext = backend.ext()
+    params, grads, exp_avgs, exp_avg_diffs, exp_avg_sqs, prev_grads, kahan_comps = _validated(
+        params, grads, (exp_avgs, exp_avg_diffs, exp_avg_sqs, prev_grads), kahan_comps)
 
     t = _tick(step)
     beta1_hat = debias_beta(beta1, t)
@@ -329,15 +352,8 @@ def adan(
     flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, ADAM_WD=adam_wd)
     scalars = (lr, 1 - beta1_hat, beta2, 1 - beta2_hat, beta3_hat, 1 - beta3_hat, eps, weight_decay, flags)
 
-    if kahan_comps is None:
-        kahan_comps = [None] * (1 if isinstance(params, Tensor) else len(params))
-    params, grads, exp_avgs, exp_avg_diffs, exp_avg_sqs, prev_grads, kahan_comps = _as_lists(
-        params, grads, exp_avgs, exp_avg_diffs, exp_avg_sqs, prev_grads, kahan_comps)
-    grads = _grads_like(params, grads)
-
     if gradient_release:
         for p, g, m, df, n, pg, k in zip(params, grads, exp_avgs, exp_avg_diffs, exp_avg_sqs, prev_grads, kahan_comps):
-            backend.check_supported(p)
             ext.adan_single(p, g, m, df, n, pg, _real_kahan(p, k), *scalars)
         return
     for (device, dtype), idxs in _buckets(params).items():
@@ -373,6 +389,11 @@ def sgd(
     """Functional API to apply a SGD or SGDW optimization step (optimi/sgd.py:213-298)."""
     _require_hip_backend(triton, foreach, gradient_release)
     ext = backend.ext()
+    if exp_avgs is None:
+        exp_avgs = [None] * (1 if isinstance(params, Tensor) else len(params))
+    # without momentum the buffer may be None or a one-element placeholder: never validated, never passed
+    params, grads, exp_avgs, kahan_comps = _validated(params, grads, (exp_avgs,), kahan_comps,
+                                                      optional=(0,) if momentum == 0 else ())
 
     if weight_decay != 0:
         if decouple_lr:
@@ -383,19 +404,11 @@ def sgd(
                    DECOUPLE_WD=decouple_wd or decouple_lr, DAMPENING=dampening)
     scalars = (lr, momentum, weight_decay, flags)
 
-    single = isinstance(params, Tensor)
-    if kahan_comps is None:
-        kahan_comps = [None] * (1 if single else len(params))
-    if exp_avgs is None:
-        exp_avgs = [None] * (1 if single else len(params))
-    params, grads, exp_avgs, kahan_comps = _as_lists(params, grads, exp_avgs, kahan_comps)
-    grads = _grads_like(params, grads)
     # without momentum the buffer is None or a one-element placeholder (optimi/sgd.py:103-106)
     moms = [_real_kahan(p, m) if momentum != 0 else None for p, m in zip(params, exp_avgs)]
 
     if gradient_release:
         for p, g, m, k in zip(params, grads, moms, kahan_comps):
-            backend.check_supported(p)
             ext.sgd_single(p, g, m, _real_kahan(p, k), *scalars)
         return
     for (device, dtype), idxs in _buckets(params).items():
@@ -443,6 +456,7 @@ def radam(
     """Functional API to apply an RAdam optimization step (optimi/radam.py:214-322)."""
     _require_hip_backend(triton, foreach, gradient_release)
     ext = backend.ext()
+    params, grads, exp_avgs, exp_avg_sqs, kahan_comps = _validated(params, grads, (exp_avgs, exp_avg_sqs), kahan_comps)
 
     t = _tick(step)
     beta1_hat = debias_beta(beta1, t)
@@ -457,14 +471,8 @@ def radam(
                    DECOUPLE_WD=decouple_wd or decouple_lr, RECTIFY=rect is not None)
     scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps, rect if rect is not None else 0.0, flags)
 
-    if kahan_comps is None:
-        kahan_comps = [None] * (1 if isinstance(params, Tensor) else len(params))
-    params, grads, exp_avgs, exp_avg_sqs, kahan_comps = _as_lists(params, grads, exp_avgs, exp_avg_sqs, kahan_comps)
-    grads = _grads_like(params, grads)
-
     if gradient_release:
         for p, g, m, v, k in zip(params, grads, exp_avgs, exp_avg_sqs, kahan_comps):
-            backend.check_supported(p)
             ext.radam_single(p, g, m, v, _real_kahan(p, k), *scalars)
         return
     for (device, dtype), idxs in _buckets(params).items():
@@ -503,6 +511,8 @@ def ranger(
     (optimi/ranger.py:230-344)."""
     _require_hip_backend(triton, foreach, gradient_release)
     ext = backend.ext()
+    params, grads, exp_avgs, exp_avg_sqs, la_params, kahan_comps = _validated(
+        params, grads, (exp_avgs, exp_avg_sqs, la_params), kahan_comps)
 
     t = _tick(step)
     beta1_hat = debias_beta(beta1, t)
@@ -517,15 +527,8 @@ def ranger(
                    DECOUPLE_WD=decouple_wd or decouple_lr, RECTIFY=rect is not None, LOOKAHEAD=t % k == 0)
     scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps, rect if rect is not None else 0.0, alpha, flags)
 
-    if kahan_comps is None:
-        kahan_comps = [None] * (1 if isinstance(params, Tensor) else len(params))
-    params, grads, exp_avgs, exp_avg_sqs, la_params, kahan_comps = _as_lists(
-        params, grads, exp_avgs, exp_avg_sqs, la_params, kahan_comps)
-    grads = _grads_like(params, grads)
-
     if gradient_release:
         for p, g, m, v, la, kc in zip(params, grads, exp_avgs, exp_avg_sqs, la_params, kahan_comps):
-            backend.check_supported(p)
             ext.ranger_single(p, g, m, v, la, _real_kahan(p, kc), *scalars)
         return
     for (device, dtype), idxs in _buckets(params).items():

@@ -422,17 +422,22 @@ class ForLoopRun:
         "ranger": dict(betas=(0.9, 0.99), weight_decay=0.0, eps=1e-6, k=6, alpha=0.5, decouple_wd=True),
     }
 
-    def __init__(self, name, params, *, gradient_release=False, **hyper):
+    def __init__(self, name, params, *, gradient_release=False, functional=False, **hyper):
         self.name = name
         self.params = list(params)
         self.gradient_release = gradient_release
+        # functional=True drives the functional form the way a direct caller does rather than the
+        # way the reference's classes do.  The one difference: Adan's ``adam_wd`` reaches the
+        # functional form (the class never forwards it, adan.py:181-203, and clears it when Kahan
+        # summation is on, adan.py:156-157).
+        self.functional = functional
         self.hyper = {**self.DEFAULTS[name], **hyper}
         if self.hyper.get("decouple_lr") and self.hyper.get("max_lr") is None:
             self.hyper["max_lr"] = self.hyper["lr"]  # optimizer.py:20-21
         ks = self.hyper.pop("kahan_sum", False if name == "adan" else None)
         self.kahan = [(ks or ks is None) and p.dtype in LOW_PRECISION for p in self.params]
         self.kahan_sum = any(self.kahan) or bool(ks)
-        if name == "adan" and self.kahan_sum:
+        if name == "adan" and self.kahan_sum and not functional:
             self.hyper["adam_wd"] = False  # adan.py:156-157
         self.state = [None] * len(self.params)
         self.group_step = torch.tensor(0, dtype=torch.int32)
@@ -473,37 +478,44 @@ class ForLoopRun:
         common = dict(step=step, kahan_sum=self.kahan_sum, optimizer_accumulation=accumulate)
         if self.name in ("adam", "adamw"):
             b1, b2 = h.pop("betas", (0.9, 0.99))
-            fn = adamw if self.name == "adamw" else adam
             if self.name == "adam":
                 h.setdefault("decouple_wd", False)
-            fn(ps, grads, col("exp_avg"), col("exp_avg_sq"), col("kahan_comp"), beta1=b1, beta2=b2, **h, **common)
+            self._invoke(self.name, [ps, grads, col("exp_avg"), col("exp_avg_sq"), col("kahan_comp")],
+                         dict(beta1=b1, beta2=b2, **h, **common))
         elif self.name == "lion":
             b1, b2 = h.pop("betas", (0.9, 0.99))
             common.pop("step")
-            lion(ps, grads, col("exp_avg"), col("kahan_comp"), beta1=b1, beta2=b2, **h, **common)
+            self._invoke("lion", [ps, grads, col("exp_avg"), col("kahan_comp")], dict(beta1=b1, beta2=b2, **h, **common))
         elif self.name == "stableadamw":
             b1, b2 = h.pop("betas", (0.9, 0.99))
-            stableadamw(ps, grads, col("exp_avg"), col("exp_avg_sq"), col("eps_sq"), col("kahan_comp"), beta1=b1,
-                        beta2=b2, **h, **common)
+            self._invoke("stableadamw", [ps, grads, col("exp_avg"), col("exp_avg_sq"), col("eps_sq"), col("kahan_comp")],
+                         dict(beta1=b1, beta2=b2, **h, **common))
         elif self.name == "adan":
             b1, b2, b3 = h.pop("betas", (0.98, 0.92, 0.99))
             # the reference class never forwards adam_wd (adan.py:181-203): always Adan-style decay
-            h.pop("adam_wd", None)
-            adan(ps, grads, col("exp_avg"), col("exp_avg_diff"), col("exp_avg_sq"), col("prev_grad"), col("kahan_comp"),
-                 beta1=b1, beta2=b2, beta3=b3, **h, **common)
+            adam_wd = bool(h.pop("adam_wd", False)) and self.functional
+            self._invoke("adan", [ps, grads, col("exp_avg"), col("exp_avg_diff"), col("exp_avg_sq"), col("prev_grad"),
+                                  col("kahan_comp")], dict(beta1=b1, beta2=b2, beta3=b3, adam_wd=adam_wd, **h, **common))
         elif self.name == "sgd":
             common.pop("step")
             h.pop("torch_init", None)
-            sgd(ps, grads, col("exp_avg"), col("kahan_comp"), **h, **common)
+            self._invoke("sgd", [ps, grads, col("exp_avg"), col("kahan_comp")], dict(**h, **common))
         elif self.name == "radam":
             b1, b2 = h.pop("betas")
-            radam(ps, grads, col("exp_avg"), col("exp_avg_sq"), col("kahan_comp"), beta1=b1, beta2=b2, **h, **common)
+            self._invoke("radam", [ps, grads, col("exp_avg"), col("exp_avg_sq"), col("kahan_comp")],
+                         dict(beta1=b1, beta2=b2, **h, **common))
         elif self.name == "ranger":
             b1, b2 = h.pop("betas")
-            ranger(ps, grads, col("exp_avg"), col("exp_avg_sq"), col("la_param"), col("kahan_comp"), beta1=b1, beta2=b2,
-                   **h, **common)
+            self._invoke("ranger", [ps, grads, col("exp_avg"), col("exp_avg_sq"), col("la_param"), col("kahan_comp")],
+                         dict(beta1=b1, beta2=b2, **h, **common))
         else:
             raise ValueError(self.name)
+
+    def _invoke(self, form, columns, kwargs):
+        """Calls the functional form ``form`` of this module on the tensor columns (params, grads, the
+        states, the Kahan buffers, in the form's positional order).  A subclass can hand the same
+        arguments to another implementation with the same signatures."""
+        globals()[form](*columns, **kwargs)
 
     def step(self, grads):
         """Whole-list step with one shared counter (adam.py:158-182).  ``grads[i] is None`` skips tensor i."""

@@ -71,11 +71,13 @@ def _beta_hat(beta: float, t: int) -> float:
     return (bt - beta) / (bt - 1)
 
 
-def step_scalars(name: str, h: dict, t: int | None, kahan_sum: bool, accumulate: bool):
+def step_scalars(name: str, h: dict, t: int | None, kahan_sum: bool, accumulate: bool, functional: bool = False):
     """The scalar arguments of one step, in the order the C entry points take them after
     ``dtype``: formed from the raw hyper-parameters ``h`` the way the reference's functional
     forms do (optimi/adam.py:260-273, lion.py:226-235, stableadamw.py:326-332, adan.py:289-309).
-    ``t`` is the already advanced step count (None for Lion)."""
+    ``t`` is the already advanced step count (None for Lion).  ``functional``: the caller is the
+    functional form itself, not a class, so Adan's ``adam_wd`` is honoured (adan.py:300-309); the
+    classes never forward it (adan.py:181-203)."""
     lr, wd = h["lr"], h.get("weight_decay", 0.0)
     flags = (KAHAN if kahan_sum else 0) | (0 if accumulate else UPDATE)
     ratio = lr / h["max_lr"] if h.get("decouple_lr") else lr  # lr, or lr/max_lr when fully decoupled
@@ -97,8 +99,11 @@ def step_scalars(name: str, h: dict, t: int | None, kahan_sum: bool, accumulate:
     if name == "adan":
         b1, b2, b3 = h.get("betas", (0.98, 0.92, 0.99))
         b1h, b2h, b3h = _beta_hat(b1, t), _beta_hat(b2, t), _beta_hat(b3, t)
-        w = 1 + ratio * wd if wd != 0 else 0.0  # the class path is always Adan-style (adan.py:181-203)
-        return (lr, 1 - b1h, b2, 1 - b2h, b3h, 1 - b3h, h["eps"], w, flags)
+        adam_wd = bool(functional and h.get("adam_wd"))  # the class path is always Adan-style (adan.py:181-203)
+        w = 0.0
+        if wd != 0:
+            w = 1 - ratio * wd if adam_wd else 1 + ratio * wd
+        return (lr, 1 - b1h, b2, 1 - b2h, b3h, 1 - b3h, h["eps"], w, flags | (ADAM_WD if adam_wd else 0))
     if name == "sgd":
         decoupled = bool(h.get("decouple_wd") or h.get("decouple_lr"))
         w = 1 - ratio * wd if (wd != 0 and decoupled) else wd
@@ -149,7 +154,7 @@ class ScalarRun(ForLoopRun):
         if self.name not in ("lion", "sgd"):
             step.add_(1)
             t = int(step.item())
-        scalars = step_scalars(self.name, self.hyper, t, self.kahan_sum, accumulate)
+        scalars = step_scalars(self.name, self.hyper, t, self.kahan_sum, accumulate, self.functional)
         fn = {"adam": L.optimi_ref_adam, "adamw": L.optimi_ref_adam, "lion": L.optimi_ref_lion,
               "stableadamw": L.optimi_ref_stableadamw, "adan": L.optimi_ref_adan, "sgd": L.optimi_ref_sgd,
               "radam": L.optimi_ref_ranger, "ranger": L.optimi_ref_ranger}[self.name]

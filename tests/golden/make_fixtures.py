@@ -41,6 +41,9 @@ RADAM = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
 # mode "group": optimizer.step() on the whole list.
 # mode "release": per-tensor step(param=p) in reverse order, accumulate-only on
 #                 micro-steps where (i+1) % 4 != 0 (optimizer accumulation).
+# mode "functional": the functional form on explicit lists of state tensors, one shared step counter.
+# mode "functional_release": the functional form on bare tensors with gradient_release=True, one
+#                 counter per tensor, reverse order, the same accumulation pattern as "release".
 CASES = {
     "adam_fp32_l2": ("Adam", dict(ADAMW, decouple_wd=False), "float32", "group", 10),
     "adam_fp32_nowd": ("Adam", dict(ADAMW, weight_decay=0.0), "float32", "group", 10),
@@ -93,18 +96,42 @@ CASES = {
     "adan_fp16_kahan_eps1e-6": ("Adan", dict(ADAN, kahan_sum=True, eps=1e-6), "float16", "group", 10),
     "sgd_fp16_kahan": ("SGD", dict(SGD, decouple_wd=True), "float16", "group", 10),
     "ranger_fp16_plain": ("Ranger", dict(RADAM, kahan_sum=False, k=3), "float16", "group", 10),
+    # Adam-style decay in Adan: only the functional form takes adam_wd (the class never forwards it,
+    # optimi/adan.py:181-203), so these cases drive optimi.adan(...) itself with explicit state lists
+    "adan_fp32_adamwd_functional": ("Adan", dict(ADAN, adam_wd=True), "float32", "functional", 10),
+    "adan_bf16_plain_adamwd_functional": ("Adan", dict(ADAN, adam_wd=True), "bfloat16", "functional", 10),
+    "adan_bf16_kahan_adamwd_functional": ("Adan", dict(ADAN, adam_wd=True, kahan_sum=True), "bfloat16", "functional", 10),
+    "adan_bf16_kahan_adamwd_declr_functional_release": (
+        "Adan", dict(ADAN, adam_wd=True, kahan_sum=True, decouple_lr=True, weight_decay=1e-3, max_lr=2e-3),
+        "bfloat16", "functional_release", 8),
 }
 
-# the first 25 cases keep the seeds they were generated with; later cases hash their name
-_FIRST_CASES = sorted(n for n in CASES if n.split("_")[0] in ("adam", "adamw", "lion", "stableadamw", "adan"))
+# The seed each committed fixture's inputs were drawn with.  Literal, so that adding a case can
+# never move another case's inputs; tests/test_oracle_golden.py regenerates every ``in.*`` array
+# from these and compares it with the stored file.
+SEEDS = {
+    "adam_bf16_kahan_l2": 1000, "adam_fp32_l2": 1001, "adam_fp32_nowd": 1002, "adamw_bf16_kahan": 1003,
+    "adamw_bf16_kahan_bigwd": 1004, "adamw_bf16_kahan_declr": 1005, "adamw_bf16_kahan_release": 1006,
+    "adamw_bf16_plain": 1007, "adamw_fp16_kahan": 1008, "adamw_fp16_kahan_release": 1009, "adamw_fp32": 1008,
+    "adamw_fp32_release": 1009, "adan_bf16_kahan": 1010, "adan_bf16_kahan_declr": 1011,
+    "adan_bf16_kahan_release": 1012, "adan_bf16_plain": 1013, "adan_fp16_kahan": 1016,
+    "adan_fp16_kahan_eps1e-6": 1017, "adan_fp32": 1014, "lion_bf16_kahan": 1015, "lion_bf16_kahan_declr": 1016,
+    "lion_bf16_kahan_release": 1017, "lion_bf16_plain": 1018, "lion_fp16_kahan": 1022, "lion_fp32": 1019,
+    "radam_bf16_kahan": 99496, "radam_bf16_kahan_release": 79847, "radam_bf16_plain_l2": 54359, "radam_fp32": 40693,
+    "ranger_bf16_kahan": 4133, "ranger_bf16_kahan_release": 39772, "ranger_bf16_plain": 92748,
+    "ranger_fp16_plain": 71565, "ranger_fp32": 78265, "sgd_bf16_kahan": 77739, "sgd_bf16_kahan_dampening": 43561,
+    "sgd_bf16_kahan_release": 79477, "sgd_bf16_plain_nomomentum": 79529, "sgd_fp16_kahan": 69834,
+    "sgd_fp32_l2": 91009, "sgd_fp32_nomomentum": 57540, "stableadamw_bf16_kahan": 1020,
+    "stableadamw_bf16_kahan_declr": 1021, "stableadamw_bf16_kahan_release": 1022, "stableadamw_bf16_plain": 1023,
+    "stableadamw_fp16_kahan": 1028, "stableadamw_fp32": 1024,
+    "adan_fp32_adamwd_functional": 3001, "adan_bf16_plain_adamwd_functional": 3002,
+    "adan_bf16_kahan_adamwd_functional": 3003, "adan_bf16_kahan_adamwd_declr_functional_release": 3004,
+}
 
 
 def case_seed(name: str) -> int:
-    if name in _FIRST_CASES:
-        return 1000 + _FIRST_CASES.index(name)
-    import zlib
+    return SEEDS[name]
 
-    return 2000 + zlib.crc32(name.encode()) % 100000
 
 STATE_KEYS = ("exp_avg", "exp_avg_sq", "exp_avg_diff", "prev_grad", "la_param", "kahan_comp")
 
@@ -179,6 +206,57 @@ def run_case(optimi, name: str, seed: int) -> dict:
     return out
 
 
+def run_functional_adan(optimi, name: str, seed: int) -> dict:
+    """Drives the reference's functional ``adan`` (optimi/adan.py:236-350), states made as the class
+    makes them (optimi/adan.py:104-120)."""
+    _, kwargs, dtype_name, mode, n_steps = CASES[name]
+    dtype = getattr(torch, dtype_name)
+    p0, grads = make_inputs(dtype, n_steps, seed)
+    out = {}
+    for i, p in enumerate(p0):
+        out[f"in.param.{i}"] = to_np(p)
+    for t, gs in enumerate(grads):
+        for i, g in enumerate(gs):
+            out[f"in.grad.{t}.{i}"] = to_np(g)
+
+    kw = dict(kwargs)
+    b1, b2, b3 = kw.pop("betas")
+    kahan = bool(kw.pop("kahan_sum", False)) and dtype != torch.float32
+    hyper = dict(lr=kw.pop("lr"), beta1=b1, beta2=b2, beta3=b3, weight_decay=kw.pop("weight_decay"), eps=kw.pop("eps"),
+                 decouple_lr=kw.pop("decouple_lr", False), max_lr=kw.pop("max_lr", None), adam_wd=kw.pop("adam_wd"),
+                 kahan_sum=kahan, foreach=False, triton=False)
+    assert not kw, kw
+    params = [p.clone() for p in p0]
+    states = [dict(exp_avg=torch.zeros_like(p), exp_avg_diff=torch.zeros_like(p), exp_avg_sq=torch.zeros_like(p),
+                   prev_grad=g.clone().mul_(-1), kahan_comp=torch.zeros_like(p) if kahan else None,
+                   step=torch.tensor(0, dtype=torch.int32)) for p, g in zip(params, grads[0])]
+    group_step = torch.tensor(0, dtype=torch.int32)
+    col = lambda key: [st[key] for st in states]  # noqa: E731
+
+    def snap(tag):
+        for i, (p, st) in enumerate(zip(params, states)):
+            out[f"{tag}.param.{i}"] = to_np(p)
+            for key in STATE_KEYS:
+                if key in st and torch.is_tensor(st[key]):
+                    out[f"{tag}.{key}.{i}"] = to_np(st[key])
+
+    for t in range(n_steps):
+        if mode == "functional_release":
+            accumulate = (t + 1) % 4 != 0
+            for i in reversed(range(len(params))):
+                st = states[i]
+                optimi.adan(params[i], grads[t][i].clone(), st["exp_avg"], st["exp_avg_diff"], st["exp_avg_sq"],
+                            st["prev_grad"], st["kahan_comp"], step=st["step"], gradient_release=True,
+                            optimizer_accumulation=accumulate, **hyper)
+        else:
+            optimi.adan(params, [g.clone() for g in grads[t]], col("exp_avg"), col("exp_avg_diff"), col("exp_avg_sq"),
+                        col("prev_grad"), col("kahan_comp") if kahan else None, step=group_step, gradient_release=False,
+                        optimizer_accumulation=False, **hyper)
+        if (t + 1) in SNAP_STEPS or t + 1 == n_steps:
+            snap(f"out.{t + 1}")
+    return out
+
+
 def main():
     ref = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
     sys.path.insert(0, ref)
@@ -189,7 +267,8 @@ def main():
     for name in sorted(CASES):
         if only and name not in only:
             continue
-        out = run_case(optimi, name, case_seed(name))
+        functional = CASES[name][3].startswith("functional")
+        out = (run_functional_adan if functional else run_case)(optimi, name, case_seed(name))
         path = os.path.join(HERE, f"{name}.npz")
         np.savez_compressed(path, **out)
         print(f"{name}: {len(out)} arrays, {os.path.getsize(path) / 1024:.1f} KiB")

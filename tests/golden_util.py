@@ -22,6 +22,8 @@ _spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(GOL
 _mk = importlib.util.module_from_spec(_spec)
 _spec.loader.exec_module(_mk)
 CASES = _mk.CASES
+SEEDS = _mk.SEEDS
+make_inputs = _mk.make_inputs
 STATE_KEYS = _mk.STATE_KEYS
 N_TENSORS = len(_mk.SHAPES)
 
@@ -42,8 +44,10 @@ def torch_tail(name: str, numel: int) -> int:
     return numel % 32 if (dtype in ("bfloat16", "float16") and uses_add_alpha) else 0
 
 
-def case_names():
-    names = sorted(CASES)
+def case_names(functional: bool | None = None):
+    """All fixture cases; ``functional`` False / True keeps only the cases written through the
+    reference's classes / through its functional form."""
+    names = sorted(n for n in CASES if functional is None or CASES[n][3].startswith("functional") == functional)
     have = {os.path.basename(p)[:-4] for p in glob.glob(os.path.join(GOLDEN_DIR, "*.npz"))}
     assert set(names) <= have, f"fixtures missing: {sorted(set(names) - have)}"
     return names
@@ -68,8 +72,10 @@ def replay(name: str, fx: dict, make_engine, device="cpu") -> dict[str, torch.Te
     """``make_engine(opt_name, params, gradient_release=..., **kwargs)`` → engine."""
     cls_name, kwargs, _dtype, mode, n_steps = CASES[name]
     params = [fx[f"in.param.{i}"].clone().to(device) for i in range(N_TENSORS)]
-    release = mode == "release"
-    eng = make_engine(OPT_NAME[cls_name], params, gradient_release=release, **kwargs)
+    release = mode in ("release", "functional_release")
+    # "functional" cases were written by the reference's functional form called directly
+    extra = {"functional": True} if mode.startswith("functional") else {}
+    eng = make_engine(OPT_NAME[cls_name], params, gradient_release=release, **extra, **kwargs)
     wanted = set(snap_steps(fx))
     out = {}
     for t in range(n_steps):

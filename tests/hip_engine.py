@@ -57,7 +57,7 @@ class HipRun(ForLoopRun):
         if self.name not in ("lion", "sgd"):
             step.add_(1)
             t = int(step.item())
-        scalars = step_scalars(self.name, self.hyper, t, self.kahan_sum, accumulate)
+        scalars = step_scalars(self.name, self.hyper, t, self.kahan_sum, accumulate, self.functional)
         sts = [self._ensure_state(i, g) for i, g in zip(idxs, grads)]
         ps = [self.params[i] for i in idxs]
         if not ps:
@@ -77,3 +77,21 @@ class HipRun(ForLoopRun):
                 bufs = [_addr(s[k]) for k in STATE_ORDER[self.name]]
                 rc = fn(*lead, _addr(p), _addr(g), *bufs, _addr(s["kahan_comp"]), p.numel(), dt, *scalars, self._stream())
                 cabi.check(rc, fn.__name__)
+
+
+class FunctionalRun(HipRun):
+    """The product's public functional forms, ``optimi_amd.adam`` ... ``optimi_amd.ranger``, called
+    the way a direct caller of the reference's functional API calls them: lists of tensors for a
+    whole-list step, bare tensors with ``gradient_release=True`` for a per-tensor step, raw
+    hyper-parameters, the int32 CPU step counter, no launch workspace of the caller's."""
+
+    def _call(self, idxs, grads, step, accumulate):
+        ForLoopRun._call(self, idxs, grads, step, accumulate)
+
+    def _invoke(self, form, columns, kwargs):
+        import optimi_amd
+
+        if self.gradient_release:  # the reference's hook hands over the tensors themselves
+            assert all(len(c) == 1 for c in columns)
+            columns = [c[0] for c in columns]
+        getattr(optimi_amd, form)(*columns, triton=True, gradient_release=self.gradient_release, **kwargs)

@@ -102,7 +102,7 @@ class ClassRun:
 
 
 @pytest.mark.parametrize("native", [True, False], ids=["native_driver", "python_driver"])
-@pytest.mark.parametrize("name", G.case_names())
+@pytest.mark.parametrize("name", G.case_names(functional=False))
 def test_fixture_through_the_optimizer_classes(name, native, hip_device):
     """Same constructor arguments and inputs as the reference was given, same bits out: the
     scalar prologue, lazy state creation and step counters of the product's Python and native
@@ -117,3 +117,19 @@ def test_fixture_through_the_optimizer_classes(name, native, hip_device):
             step, _, idx = key.split(".")[1:4]
             param_key = f"out.{step}.param.{idx}"
         compare_snapshot(name, key, out[key], fx[key], fx[param_key] if param_key else None)
+
+
+@pytest.mark.parametrize("name", G.case_names())
+def test_fixture_through_the_functional_forms(name, hip_device):
+    """The eight public functional forms called directly, as the reference's functional API is
+    called: lists for whole-list cases, bare tensors with ``gradient_release=True`` for release
+    cases, no workspace passed in.  Same bar as the kernels."""
+    from hip_engine import FunctionalRun
+
+    fx = G.load(name)
+    out = G.replay(name, fx, FunctionalRun, device=hip_device)
+    wanted = [k for k in fx if k.startswith("out.")]
+    assert sorted(out) == sorted(wanted)
+    for key in wanted:
+        step, _, idx = key.split(".")[1:4]
+        compare_snapshot(name, key, out[key], fx[key], fx.get(f"out.{step}.param.{idx}"))

@@ -102,12 +102,34 @@ def test_functional_forms_refuse_other_backends():
         F.adamw([p], [g], [m], [v], **kw)
     with pytest.raises(RuntimeError, match="HIP devices only"):  # foreach=True selects the HIP kernels too
         F.adamw([p], [g], [m], [v], foreach=True, **kw)
-    step.zero_()
     with pytest.raises(ValueError, match="cannot be used together"):
         F.adamw(p, g, m, v, foreach=True, gradient_release=True, **kw)
-    assert int(step) == 0  # rejected before the counter moved
     with pytest.raises(RuntimeError, match="HIP devices only"):
         F.adamw([p], [g], [m], [v], triton=True, **kw)
+    assert int(step) == 0  # every rejected call left the counter where it was
+
+
+def test_rejected_calls_do_not_advance_the_step_counter():
+    """Tensors are validated before the counter moves, in every functional form that has one."""
+    p, g, m, v, x, y = (torch.zeros(4) for _ in range(6))
+    base = dict(lr=1e-3, beta1=0.9, beta2=0.99, weight_decay=0.0, eps=1e-6, triton=True)
+    calls = {
+        "adam": lambda s: F.adam([p], [g], [m], [v], decouple_wd=True, step=s, **base),
+        "stableadamw": lambda s: F.stableadamw([p], [g], [m], [v], [x], step=s, **base),
+        "adan": lambda s: F.adan([p], [g], [m], [v], [x], [y], beta3=0.99, step=s, **base),
+        "radam": lambda s: F.radam([p], [g], [m], [v], decouple_wd=True, step=s, **base),
+        "ranger": lambda s: F.ranger([p], [g], [m], [v], [x], k=6, alpha=0.5, decouple_wd=True, step=s, **base),
+    }
+    for name, call in calls.items():
+        step = torch.tensor(3, dtype=torch.int32)
+        with pytest.raises(RuntimeError, match="HIP devices only"):
+            call(step)
+        assert int(step) == 3, name
+    # a gradient of another dtype and lists of unequal length are rejected before the counter moves, too
+    step = torch.tensor(3, dtype=torch.int32)
+    with pytest.raises(ValueError, match="got 1 parameters but a list of 2"):
+        F.adam([p], [g, g], [m], [v], decouple_wd=True, step=step, **base)
+    assert int(step) == 3
 
 
 def test_step_without_gradients_is_a_noop_that_still_counts():

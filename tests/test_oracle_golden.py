@@ -49,3 +49,20 @@ def test_scalar_emulator(name):
         else:
             rel = G.fp32_rel_err(got, want, 1e-2)
             assert float(rel.max()) <= 1e-6, f"{name} {k}: rel err {float(rel.max())}"
+
+
+@pytest.mark.parametrize("name", G.case_names())
+def test_committed_recipe_regenerates_the_fixture_inputs(name):
+    """``make_fixtures.make_inputs`` with the frozen seed of the case reproduces every stored
+    ``in.*`` array, so the committed script and the committed files belong together (the outputs
+    need the reference; the inputs do not)."""
+    _cls, _kwargs, dtype_name, _mode, n_steps = G.CASES[name]
+    fx = G.load(name)
+    params, grads = G.make_inputs(getattr(torch, dtype_name), n_steps, G.SEEDS[name])
+    stored = sorted(k for k in fx if k.startswith("in."))
+    assert len(stored) == len(params) * (1 + n_steps)
+    for i, p in enumerate(params):
+        assert torch.equal(bits(p), bits(fx[f"in.param.{i}"])), f"{name} in.param.{i}"
+    for t, gs in enumerate(grads):
+        for i, g in enumerate(gs):
+            assert torch.equal(bits(g), bits(fx[f"in.grad.{t}.{i}"])), f"{name} in.grad.{t}.{i}"

@@ -34,7 +34,7 @@ def draw_config(seed):
     if name == "sgd":
         h.update(momentum=rnd.choice([0.0, 0.4, 0.9]), dampening=rnd.random() < 0.4, torch_init=rnd.random() < 0.3)
     elif name == "adan":
-        h.update(betas=(beta(), beta(), beta()))
+        h.update(betas=(beta(), beta(), beta()), adam_wd=rnd.random() < 0.5)
     else:
         h.update(betas=(beta(), beta()))
     if name not in ("lion", "sgd"):
@@ -53,6 +53,12 @@ def draw_config(seed):
         h.update(kahan_sum=rnd.random() < 0.6)
     release = rnd.random() < 0.4
     return name, dtype, h, release, rnd.randrange(1 << 30)
+
+
+def engine_mode(name, hyper):
+    """Adan's Adam-style decay exists in the functional form only: those configurations drive the
+    engines as a direct caller of the functional form would."""
+    return dict(functional=True) if (name == "adan" and hyper.get("adam_wd")) else {}
 
 
 def draw_tensors(dtype, seed, steps):
@@ -78,8 +84,9 @@ def test_emulator_matches_forloop(seed):
     name, dtype, hyper, release, data_seed = draw_config(seed)
     torch.set_num_threads(1)
     params, grads = draw_tensors(dtype, data_seed, 7)
-    sca = ScalarRun(name, [p.clone() for p in params], gradient_release=release, **hyper)
-    ref = ForLoopRun(name, [p.clone() for p in params], gradient_release=release, **hyper)
+    mode = engine_mode(name, hyper)
+    sca = ScalarRun(name, [p.clone() for p in params], gradient_release=release, **mode, **hyper)
+    ref = ForLoopRun(name, [p.clone() for p in params], gradient_release=release, **mode, **hyper)
     drive([(sca, torch.clone), (ref, torch.clone)], grads, release)
     what = f"seed {seed}: {name} {dtype} {hyper} release={release}"
     if dtype == torch.float32:
@@ -95,7 +102,8 @@ def test_hip_matches_emulator(seed, hip_device):
 
     name, dtype, hyper, release, data_seed = draw_config(seed)
     params, grads = draw_tensors(dtype, data_seed, 7)
-    hip = HipRun(name, [p.to(hip_device) for p in params], gradient_release=release, **hyper)
-    sca = ScalarRun(name, [p.clone() for p in params], gradient_release=release, **hyper)
+    mode = engine_mode(name, hyper)
+    hip = HipRun(name, [p.to(hip_device) for p in params], gradient_release=release, **mode, **hyper)
+    sca = ScalarRun(name, [p.clone() for p in params], gradient_release=release, **mode, **hyper)
     drive([(hip, lambda g: g.to(hip_device)), (sca, torch.clone)], grads, release)
     G.compare_engines(hip, sca, f"seed {seed}: {name} {dtype} {hyper} release={release}", exact=name != "stableadamw")
