@@ -277,6 +277,42 @@ def test_coalesced_release_equals_per_tensor_launches(case, max_tensors, hip_dev
     optimi_amd.remove_gradient_release(b)
 
 
+def test_release_flush_is_ordered_before_the_callers_next_work(hip_device):
+    """Forward on a side stream, backward() called on the default stream: the autograd engine
+    runs the hooks on the side stream (where the parameters were used) and makes the default
+    stream wait for it before the final callbacks run.  The flush of the parked steps happens in
+    such a callback; work the caller enqueues on the default stream right after backward() - here
+    a copy of every parameter - must see its result.  The side stream is kept busy so that a
+    flush left on it would still be waiting when the copies run."""
+    a, b = ManySmall(hip_device), ManySmall(hip_device)
+    hyper = CASES["adamw"][2]
+    parked = optimi_amd.AdamW(a.parameters(), gradient_release=True, **hyper)
+    direct = optimi_amd.AdamW(b.parameters(), gradient_release=True, **hyper)
+    direct.gradient_release_coalesce = 0
+    optimi_amd.prepare_for_gradient_release(a, parked)
+    optimi_amd.prepare_for_gradient_release(b, direct)
+    side = torch.cuda.Stream()
+    ballast = torch.randn(4096, 4096, device=hip_device)
+    torch.cuda.synchronize()
+    for it in range(6):
+        snaps = []
+        for model in (a, b):
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                loss = model(1.0 + it)
+                for _ in range(8):
+                    ballast @ ballast  # keeps the side stream busy past the end of backward()
+            loss.backward()
+            snaps.append([p.detach().clone() for p in model.parameters()])  # default stream, no sync in between
+        assert parked._release_queue.pending() == 0
+        torch.cuda.synchronize()
+        for i, (x, y) in enumerate(zip(*snaps)):
+            G.assert_bits_equal(x, y, f"pass {it} param {i} as the default stream saw it right after backward()")
+    assert not torch.equal(next(a.parameters()), ManySmall(hip_device).ps[0]), "nothing was stepped"
+    optimi_amd.remove_gradient_release(a)
+    optimi_amd.remove_gradient_release(b)
+
+
 def test_release_outside_a_backward_pass_launches_at_once(hip_device):
     """Steps are parked only inside a backward pass (its end launches them); a hook body called
     by hand launches its tensor directly."""
