@@ -57,7 +57,8 @@ enum optimi_status {
   OPTIMI_ERR_ALIGN = -4,     /* a buffer is not aligned to its element size        */
   OPTIMI_ERR_DEVICE = -5,    /* group used on a device other than the one it was made on */
   OPTIMI_ERR_NOMEM = -6,     /* host allocation failed                             */
-  OPTIMI_ERR_ARG = -7        /* inconsistent scalar argument (e.g. max_lr <= 0 with OPTIMI_DECOUPLE_LR) */
+  OPTIMI_ERR_ARG = -7,       /* inconsistent scalar argument (e.g. max_lr <= 0 with OPTIMI_DECOUPLE_LR) */
+  OPTIMI_ERR_LIMIT = -8      /* numel above OPTIMI_NOALLOC_MAX_NUMEL in the allocation-free entry point */
 };
 
 /* Text for a status returned by any function of this header. */
@@ -170,6 +171,24 @@ int optimi_hip_stableadamw_single(optimi_group* group, void* param, const void* 
                                   void* kahan_comp, int64_t numel, int dtype, double lr, double beta1_comp,
                                   double beta2_hat, double beta2_comp, double weight_decay, double eps, double max_lr,
                                   uint32_t flags, optimi_stream_t stream);
+
+/* The same step as optimi_hip_stableadamw_single for callers that cannot allocate: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference.  It takes no group: the reduction partials and the
+ * per-tensor scalars live in a fixed array of OPTIMI_NOALLOC_SCRATCH_BYTES that is part of
+ * the library's device code (one copy per GPU, held until the process ends), so the call
+ * makes no hipMalloc/hipFree and no other allocating call; the first call on a device only
+ * looks the array's address up (hipGetSymbolAddress), so make one call outside a capture first.
+ * A tensor with more than OPTIMI_NOALLOC_MAX_NUMEL(dtype) elements is rejected with
+ * OPTIMI_ERR_LIMIT.  Every call on a GPU uses that GPU's one array: calls that may overlap
+ * on one GPU (different streams, different threads) race and must be ordered by the caller.
+ * Results are bit-identical to optimi_hip_stableadamw_single. */
+#define OPTIMI_NOALLOC_SCRATCH_BYTES (4u * 1024u * 1024u + 256u)
+#define OPTIMI_NOALLOC_MAX_NUMEL(dtype) ((dtype) == OPTIMI_F32 ? (int64_t)134217728 : (int64_t)268435456)
+int optimi_hip_stableadamw_single_noalloc(void* param, const void* grad, void* exp_avg, void* exp_avg_sq,
+                                          void* kahan_comp, int64_t numel, int dtype, double lr, double beta1_comp,
+                                          double beta2_hat, double beta2_comp, double weight_decay, double eps,
+                                          double max_lr, uint32_t flags, optimi_stream_t stream);
 
 /* Replaces _single_param_triton_adan (optimi/adan.py:713-770). */
 int optimi_hip_adan_single(void* param, const void* grad, void* exp_avg, void* exp_avg_diff, void* exp_avg_sq,

@@ -35,6 +35,7 @@ PROTOTYPES = {
     "optimi_hip_adam_single": (_i, [_p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_lion_single": (_i, [_p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_stableadamw_single": (_i, [_p, _p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_stableadamw_single_noalloc": (_i, [_p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_adan_single": (_i, [_p, _p, _p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_sgd_single": (_i, [_p, _p, _p, _p, _i64, _i, _d, _d, _d, _u32, _p]),
     "optimi_hip_radam_single": (_i, [_p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),

@@ -25,6 +25,7 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <type_traits>
 #include <vector>
@@ -942,11 +943,11 @@ unsigned throttle_lds(int64_t workgroups) {
 }
 
 template <class Op>
-void launch_multi(optimi_group* g, const typename Op::Scalars& s, hipStream_t stream) {
+void launch_multi(optimi_group* g, const typename Op::Scalars& s, hipStream_t stream, double* partials = nullptr) {
   TensorEntry none;
   std::memset(&none, 0, sizeof(none));
   step_kernel<Op, true><<<dim3((unsigned)(g->n_chunks * kSub)), dim3(kThreads), throttle_lds<Op>(g->n_chunks * kSub), stream>>>(
-      (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, none, s, (double*)g->partials.ptr);
+      (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, none, s, partials);
 }
 
 template <class Op>
@@ -1138,55 +1139,122 @@ inline bool kahan_on(int dtype, uint32_t flags) {
   return dtype != OPTIMI_F32 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
 }
 
+// The device scratch one StableAdamW step needs beyond the caller's tensors: one double per
+// pass-1 workgroup and the per-tensor scalars the finalize kernel hands to pass 2.
+struct StableScratch {
+  double* partials;
+  TensorScalars* tensor_scalars;
+};
+
 template <class DT>
-int stable_run(bool multi, optimi_group* g, const TensorEntry& single, int n_tensors, int dtype, double lr,
-               double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay, double eps, double max_lr,
-               uint32_t flags, hipStream_t stream) {
+int64_t stable_partials(int64_t numel) {  // pass-1 workgroups of one tensor
+  const int64_t chunk = chunk_elems<DT>();
+  return (numel + chunk - 1) / chunk * kSub;
+}
+
+// `scratch` is written before it is read within the call (every pass-1 workgroup stores its
+// partial, finalize stores the scalars), so it needs no clearing between calls.
+template <class DT>
+int stable_run(bool multi, optimi_group* g, const TensorEntry& single, int n_tensors, const StableScratch& scratch,
+               int dtype, double lr, double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay,
+               double eps, double max_lr, uint32_t flags, hipStream_t stream) {
   const bool update = (flags & OPTIMI_UPDATE) != 0;
   const bool kahan = kahan_on(dtype, flags);
-  const int64_t chunk = chunk_elems<DT>();
-  const int64_t n_chunks = multi ? g->n_chunks : (single.numel + chunk - 1) / chunk;
-  if (n_chunks == 0) return 0;
   StableP1Scalars s1 = stable_p1_scalars(dtype, beta1_comp, beta2_hat, beta2_comp, eps);
   if (!update) {
     if (multi) launch_multi<StablePass1Op<DT, false>>(g, s1, stream);
     else launch_single<StablePass1Op<DT, false>>(single, s1, nullptr, stream);
     return 0;
   }
-  int rc = g->partials.reserve(sizeof(double) * (size_t)n_chunks * kSub);
-  if (rc) return rc;
-  rc = g->tensor_scalars.reserve(sizeof(TensorScalars) * (size_t)(multi ? n_tensors : 1));
-  if (rc) return rc;
   FinalizeArgs fa;
   fa.lr = lr;
   fa.weight_decay = weight_decay;
   fa.max_lr = max_lr;
   fa.decouple_lr = (flags & OPTIMI_DECOUPLE_LR) ? 1u : 0u;
   StableP2Scalars s2;
-  s2.per_tensor = (const TensorScalars*)g->tensor_scalars.ptr;
+  s2.per_tensor = scratch.tensor_scalars;
   s2.eps_d = Sd(eps, dtype);
   s2.neg_lr = 0.0f;
   s2.wd = 0.0f;
   const bool wd = weight_decay != 0;
   if (multi) {
-    launch_multi<StablePass1Op<DT, true>>(g, s1, stream);
+    launch_multi<StablePass1Op<DT, true>>(g, s1, stream, scratch.partials);
     TensorEntry none;
     std::memset(&none, 0, sizeof(none));
     stable_finalize_kernel<DT, true><<<dim3((unsigned)n_tensors), dim3(kReduceThreads), 0, stream>>>(
-        (const TensorEntry*)g->table.ptr, none, (const double*)g->partials.ptr, (TensorScalars*)g->tensor_scalars.ptr, fa);
+        (const TensorEntry*)g->table.ptr, none, scratch.partials, scratch.tensor_scalars, fa);
     if (kahan && wd) launch_multi<StablePass2Op<DT, true, 1>>(g, s2, stream);
     else if (kahan) launch_multi<StablePass2Op<DT, true, 0>>(g, s2, stream);
     else if (wd) launch_multi<StablePass2Op<DT, false, 1>>(g, s2, stream);
     else launch_multi<StablePass2Op<DT, false, 0>>(g, s2, stream);
   } else {
-    launch_single<StablePass1Op<DT, true>>(single, s1, (double*)g->partials.ptr, stream);
+    launch_single<StablePass1Op<DT, true>>(single, s1, scratch.partials, stream);
     stable_finalize_kernel<DT, false><<<dim3(1), dim3(kReduceThreads), 0, stream>>>(
-        nullptr, single, (const double*)g->partials.ptr, (TensorScalars*)g->tensor_scalars.ptr, fa);
+        nullptr, single, scratch.partials, scratch.tensor_scalars, fa);
     if (kahan && wd) launch_single<StablePass2Op<DT, true, 1>>(single, s2, nullptr, stream);
     else if (kahan) launch_single<StablePass2Op<DT, true, 0>>(single, s2, nullptr, stream);
     else if (wd) launch_single<StablePass2Op<DT, false, 1>>(single, s2, nullptr, stream);
     else launch_single<StablePass2Op<DT, false, 0>>(single, s2, nullptr, stream);
   }
+  return 0;
+}
+
+// The group's own scratch, grown to what this step needs (whole list: `multi`; else one tensor).
+template <class DT>
+int group_scratch(optimi_group* g, bool multi, int64_t single_numel, int n_tensors, uint32_t flags, StableScratch* out) {
+  out->partials = nullptr;
+  out->tensor_scalars = nullptr;
+  if (!(flags & OPTIMI_UPDATE)) return 0;  // the accumulate-only step reduces nothing
+  const int64_t n_partials = multi ? g->n_chunks * kSub : stable_partials<DT>(single_numel);
+  int rc = g->partials.reserve(sizeof(double) * (size_t)n_partials);
+  if (rc) return rc;
+  rc = g->tensor_scalars.reserve(sizeof(TensorScalars) * (size_t)(multi ? n_tensors : 1));
+  if (rc) return rc;
+  out->partials = (double*)g->partials.ptr;
+  out->tensor_scalars = (TensorScalars*)g->tensor_scalars.ptr;
+  return 0;
+}
+
+template <class DT>
+int stable_group_run(bool multi, optimi_group* g, const TensorEntry& single, int n_tensors, int dtype, double lr,
+                     double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay, double eps,
+                     double max_lr, uint32_t flags, hipStream_t stream) {
+  StableScratch scratch;
+  int rc = group_scratch<DT>(g, multi, single.numel, n_tensors, flags, &scratch);
+  if (rc) return rc;
+  return stable_run<DT>(multi, g, single, n_tensors, scratch, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay,
+                        eps, max_lr, flags, stream);
+}
+
+// ---- fixed scratch of the allocation-free entry point ---------------------------------------
+// One array per GPU, part of the loaded code object, so it exists from the moment the library
+// is loaded on a device until the process ends and no call ever allocates it.  Layout: the
+// per-tensor scalars in the first 256 bytes, then the pass-1 partials.  `scratch` itself is only
+// a host-side handle for hipGetSymbolAddress; kernels get the address that call returns for the
+// device they run on.
+constexpr size_t kScratchHead = 256;
+constexpr size_t kScratchBytes = OPTIMI_NOALLOC_SCRATCH_BYTES;
+constexpr int64_t kScratchPartials = (int64_t)((kScratchBytes - kScratchHead) / sizeof(double));
+static_assert(kScratchBytes % 256 == 0 && sizeof(TensorScalars) <= kScratchHead, "scratch layout");
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_addr[kMaxDevices] = {};
+
+// Address of the current device's copy of `scratch`; resolved once per device.
+int device_scratch(void** out) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return OPTIMI_ERR_DEVICE;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_addr[dev]) {
+    void* p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p || ((uintptr_t)p % 256)) return OPTIMI_ERR_ALIGN;
+    scratch_addr[dev] = p;
+  }
+  *out = scratch_addr[dev];
   return 0;
 }
 
@@ -1207,6 +1275,7 @@ const char* optimi_hip_error_string(int status) {
     case OPTIMI_ERR_DEVICE: return "optimi_hip: group used on a different device than it was created on";
     case OPTIMI_ERR_NOMEM: return "optimi_hip: host allocation failed";
     case OPTIMI_ERR_ARG: return "optimi_hip: inconsistent scalar argument";
+    case OPTIMI_ERR_LIMIT: return "optimi_hip: tensor has more elements than the fixed scratch of the allocation-free entry point covers (OPTIMI_NOALLOC_MAX_NUMEL)";
     default: break;
   }
   if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -1301,10 +1370,10 @@ int optimi_hip_stableadamw_multi(optimi_group* g, int n_tensors, void* const* pa
   TensorEntry none;
   std::memset(&none, 0, sizeof(none));
   rc = dtype == OPTIMI_BF16
-           ? stable_run<BF16>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           ? stable_group_run<BF16>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
        : dtype == OPTIMI_F16
-           ? stable_run<F16>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
-           : stable_run<F32>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
+           ? stable_group_run<F16>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           : stable_group_run<F32>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
   if (rc) return rc;
   return note_launch(g, stream);
 }
@@ -1377,12 +1446,43 @@ int optimi_hip_stableadamw_single(optimi_group* g, void* param, const void* grad
   if (dev != g->device) return OPTIMI_ERR_DEVICE;
   if (g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
   rc = dtype == OPTIMI_BF16
-           ? stable_run<BF16>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           ? stable_group_run<BF16>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
        : dtype == OPTIMI_F16
-           ? stable_run<F16>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
-           : stable_run<F32>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
+           ? stable_group_run<F16>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           : stable_group_run<F32>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
   if (rc) return rc;
   return note_launch(g, stream);
+}
+
+int optimi_hip_stableadamw_single_noalloc(void* param, const void* grad, void* exp_avg, void* exp_avg_sq,
+                                          void* kahan_comp, int64_t numel, int dtype, double lr, double beta1_comp,
+                                          double beta2_hat, double beta2_comp, double weight_decay, double eps,
+                                          double max_lr, uint32_t flags, optimi_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if ((flags & OPTIMI_DECOUPLE_LR) && weight_decay != 0 && !(max_lr > 0)) return OPTIMI_ERR_ARG;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const void* ptrs[5] = {param, grad, exp_avg, exp_avg_sq, kahan_comp};
+  TensorEntry e;
+  int rc = single_entry(e, ptrs, 5, adam_need(kahan, update), numel, dtype);
+  if (rc) return rc;
+  if (numel > OPTIMI_NOALLOC_MAX_NUMEL(dtype)) return OPTIMI_ERR_LIMIT;
+  if (numel == 0) return 0;
+  void* base = nullptr;
+  rc = device_scratch(&base);
+  if (rc) return rc;
+  StableScratch sc;
+  sc.tensor_scalars = (TensorScalars*)base;
+  sc.partials = (double*)((unsigned char*)base + kScratchHead);
+  const int64_t n_partials = dtype == OPTIMI_F32 ? stable_partials<F32>(numel) : stable_partials<BF16>(numel);
+  if (n_partials > kScratchPartials) return OPTIMI_ERR_LIMIT;  // the macro and the layout must agree
+  rc = dtype == OPTIMI_BF16
+           ? stable_run<BF16>(false, nullptr, e, 1, sc, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+       : dtype == OPTIMI_F16
+           ? stable_run<F16>(false, nullptr, e, 1, sc, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           : stable_run<F32>(false, nullptr, e, 1, sc, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
+  if (rc) return rc;
+  HIP_TRY(hipGetLastError());
+  return 0;
 }
 
 int optimi_hip_adan_single(void* param, const void* grad, void* exp_avg, void* exp_avg_diff, void* exp_avg_sq,

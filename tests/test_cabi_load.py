@@ -30,7 +30,7 @@ def test_error_strings_and_constants():
     L = cabi.lib()
     assert L.optimi_hip_version() >= 1000
     assert L.optimi_hip_error_string(0) == b"success"
-    for code in range(-7, 0):
+    for code in range(-8, 0):
         msg = L.optimi_hip_error_string(code)
         assert msg.startswith(b"optimi_hip:"), (code, msg)
     assert L.optimi_hip_chunk_elems(cabi.BF16) == 8192
