@@ -58,8 +58,15 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 // Pointers come out of the tensor table as plain addresses; telling the compiler they are
 // global memory gets global_load/global_store instead of flat accesses.
 #define OPTIMI_GLOBAL __attribute__((address_space(1)))
+#ifndef OPTIMI_LOAD_NT
+#define OPTIMI_LOAD_NT 1  // 16-byte loads carry the `nt` policy (tuning builds set 0 to compare)
+#endif
 __device__ __forceinline__ u32x4 load16(const void* base, int64_t byte_off) {
+#if OPTIMI_LOAD_NT
   return __builtin_nontemporal_load((const OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
+#else
+  return *(const OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off);
+#endif
 }
 __device__ __forceinline__ void store16(void* base, int64_t byte_off, u32x4 v) {
   __builtin_nontemporal_store(v, (OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
@@ -72,7 +79,10 @@ __device__ __forceinline__ void store16(void* base, int64_t byte_off, u32x4 v) {
 // express the policy, the buffer builtin can, and unlike inline assembly it is tracked by the
 // compiler's wait-count insertion.  `tile` (wave-uniform) points at the workgroup's tile of
 // one array, `lane_off` is the lane's byte offset in it.
-constexpr int kStorePolicy = 1 | 16;  // aux bits of the buffer instructions on gfx94x/gfx950: 1 sc0, 2 nt, 16 sc1
+#ifndef OPTIMI_STORE_POLICY
+#define OPTIMI_STORE_POLICY (1 | 16)
+#endif
+constexpr int kStorePolicy = OPTIMI_STORE_POLICY;  // aux bits of the buffer instructions on gfx94x/gfx950: 1 sc0, 2 nt, 16 sc1
 __device__ __forceinline__ void store16_tile(void* tile, uint32_t lane_off, u32x4 v) {
   // dword 3 = 0x00020000: raw buffer, 32-bit data format; stride 0; bounds = the tile
   __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(tile, 0, (uint32_t)(kThreads * kUnroll * 16), 0x00020000);
@@ -931,6 +941,9 @@ unsigned throttle_lds(int64_t workgroups) {
   constexpr bool f32 = std::is_same<typename Op::DT, F32>::value;
   int waves = kBestWaves[streams < kMaxStreams ? streams : kMaxStreams] + ((f32 && streams == 7) ? 1 : 0);
   if (workgroups * (kThreads / 64) < (int64_t)kShortRounds * kCus * waves && waves < kShortWaves) waves = kShortWaves;
+#ifdef OPTIMI_TUNING
+  if (const char* env = std::getenv("OPTIMI_HIP_LDS")) return (unsigned)std::strtol(env, nullptr, 10);  // raw request, tuning builds only
+#endif
   const int forced = forced_waves();
   if (forced == 0) return 0;
   if (forced > 0) waves = forced;

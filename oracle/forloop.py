@@ -22,7 +22,9 @@ function                   pinned by
                            scalar C emulator bit-equality
 ``stableadamw_tensor``     golden fixtures; rms<=1 reduces to ``adam_tensor``;
                            scalar C emulator
-``adan_tensor``            golden fixtures; t=1 closed form; scalar C emulator
+``adan_tensor``            golden fixtures (class path, and the functional form with
+                           ``adam_wd=True``); t=1 closed form; float64 textbook Adan in
+                           both decay styles; scalar C emulator
 ``sgd_tensor``             golden fixtures; torch.optim.SGD equivalence in fp32;
                            scalar C emulator
 ``radam_tensor``           golden fixtures; torch.optim.RAdam equivalence in fp32;

@@ -90,7 +90,7 @@ def test_fully_decoupled_lr_equals_rescaled_adamw(engine):
         torch.testing.assert_close(eng.params[i], p.detach(), rtol=1e-5, atol=1e-6)
 
 
-def textbook(name, params, grads, *, lr, betas, eps=0.0, wd=0.0):
+def textbook(name, params, grads, *, lr, betas, eps=0.0, wd=0.0, adam_wd=False):
     """float64, raw EMAs, explicit bias corrections."""
     out = []
     for i, p0 in enumerate(params):
@@ -117,7 +117,10 @@ def textbook(name, params, grads, *, lr, betas, eps=0.0, wd=0.0):
                 d = b2 * d + (1 - b2) * diff
                 v = b3 * v + (1 - b3) * (g + b2 * diff) ** 2
                 mh, dh, vh = m / (1 - b1**t), d / (1 - b2**t), v / (1 - b3**t)
-                p = (p - lr * (mh + b2 * dh) / (np.sqrt(vh) + eps)) / (1 + lr * wd)
+                if adam_wd:  # decay the weights first, Adam style, instead of Adan's division after the step
+                    p = p * (1 - lr * wd) - lr * (mh + b2 * dh) / (np.sqrt(vh) + eps)
+                else:
+                    p = (p - lr * (mh + b2 * dh) / (np.sqrt(vh) + eps)) / (1 + lr * wd)
                 prev = g
         out.append(p)
     return out
@@ -138,6 +141,134 @@ def test_matches_textbook_algorithm(engine, name, hyper):
         bad = np.abs(got - w) > 1e-6 + 1e-5 * np.abs(w)
         # Lion: sign() of a value within rounding of zero may legitimately flip; nothing else may differ
         assert bad.sum() <= (2 if name == "lion" else 0), f"{name} tensor {i}: {bad.sum()} elements off, max {np.abs(got - w).max()}"
+
+
+@pytest.mark.parametrize("engine", ENGINES)
+def test_adan_adam_style_decay_matches_textbook(engine):
+    """``adam_wd=True`` reaches the functional form only (``functional=True`` drives the engines that
+    way): weights decay by 1 - lr*wd before the step.  A large decay makes the two styles differ
+    far beyond the tolerance, so taking the wrong branch fails."""
+    hyper = dict(lr=1e-3, betas=(0.98, 0.92, 0.99), eps=1e-8, weight_decay=5.0)
+    params, grads = draw(14)
+    eng = engine("adan", [p.clone() for p in params], functional=True, adam_wd=True, **hyper)
+    cls_style = engine("adan", [p.clone() for p in params], adam_wd=True, **hyper)  # as a class: the flag is dropped
+    for gs in grads:
+        eng.step([g.clone() for g in gs])
+        cls_style.step([g.clone() for g in gs])
+    for style, e in ((True, eng), (False, cls_style)):
+        want = textbook("adan", params, grads, lr=hyper["lr"], betas=hyper["betas"], eps=hyper["eps"], wd=5.0, adam_wd=style)
+        for i, w in enumerate(want):
+            got = e.params[i].double().numpy()
+            assert (np.abs(got - w) <= 1e-6 + 1e-5 * np.abs(w)).all(), f"adam_wd={style} tensor {i}"
+    assert not torch.allclose(eng.params[0], cls_style.params[0], rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("engine", ENGINES)
+@pytest.mark.parametrize("variant", ["momentum_l2", "dampening_torch_init", "plain_decoupled"])
+def test_sgd_equals_torch_optim(engine, variant):
+    """fp32 SGD is torch.optim.SGD up to rounding (the reference's own comparison, tests/opt_sgd.py).
+    ``dampening=True`` makes the buffer an EMA, m = momentum*m + (1 - momentum)*g, which is torch's
+    ``dampening = momentum`` once the buffer starts from the first gradient (``torch_init``);
+    decoupled decay multiplies the parameter by 1 - lr*wd before the step, which for plain SGD is
+    torch's L2 decay with the same coefficient up to the lr^2 term - so that variant is checked
+    against an explicit float64 recursion instead."""
+    lr, mu, wd = 1e-2, 0.9, 1e-2
+    params, grads = draw(11)
+    tp = [torch.nn.Parameter(p.clone()) for p in params]
+    if variant == "momentum_l2":
+        eng = run(engine, "sgd", params, grads, lr=lr, momentum=mu, weight_decay=wd)
+        topt = torch.optim.SGD(tp, lr=lr, momentum=mu, weight_decay=wd, foreach=False)
+    elif variant == "dampening_torch_init":
+        eng = run(engine, "sgd", params, grads, lr=lr, momentum=mu, weight_decay=wd, dampening=True, torch_init=True)
+        topt = torch.optim.SGD(tp, lr=lr, momentum=mu, dampening=mu, weight_decay=wd, foreach=False)
+    else:
+        eng = run(engine, "sgd", params, grads, lr=lr, momentum=0.0, weight_decay=wd, decouple_wd=True)
+        for i, p0 in enumerate(params):
+            p = p0.double()
+            for gs in grads:
+                p = p * (1 - lr * wd) - lr * gs[i].double()
+            torch.testing.assert_close(eng.params[i].double(), p, rtol=1e-5, atol=1e-7)
+            assert eng.state[i]["exp_avg"] is None
+        return
+    for gs in grads:
+        for p, g in zip(tp, gs):
+            p.grad = g.clone()
+        topt.step()
+    for i, p in enumerate(tp):
+        torch.testing.assert_close(eng.params[i], p.detach(), rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(eng.state[i]["exp_avg"], topt.state[p]["momentum_buffer"], rtol=1e-5, atol=1e-8)
+
+
+@pytest.mark.parametrize("engine", ENGINES)
+@pytest.mark.parametrize("decoupled", [True, False])
+def test_radam_equals_torch_optim(engine, decoupled):
+    """fp32 RAdam is torch.optim.RAdam up to rounding and the place of eps (torch adds it to
+    sqrt(v) before the bias correction, the reference after: with eps = 1e-12 the two agree far
+    below the tolerance).  14 steps at beta2 = 0.99 cover the unrectified steps (t <= 5) and the
+    rectified ones.  The debiased moments map to torch's raw ones as for Adam."""
+    lr, betas, eps, wd = 1e-3, (0.9, 0.99), 1e-12, 1e-2
+    params, grads = draw(12, steps=14)
+    eng = run(engine, "radam", params, grads, lr=lr, betas=betas, eps=eps, weight_decay=wd, decouple_wd=decoupled)
+    tp = [torch.nn.Parameter(p.clone()) for p in params]
+    topt = torch.optim.RAdam(tp, lr=lr, betas=betas, eps=eps, weight_decay=wd, decoupled_weight_decay=decoupled, foreach=False)
+    for gs in grads:
+        for p, g in zip(tp, gs):
+            p.grad = g.clone()
+        topt.step()
+    t = len(grads)
+    for i, p in enumerate(tp):
+        torch.testing.assert_close(eng.params[i], p.detach(), rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(eng.state[i]["exp_avg"], topt.state[p]["exp_avg"] / (1 - betas[0] ** t), rtol=1e-5, atol=1e-9)
+        torch.testing.assert_close(eng.state[i]["exp_avg_sq"], topt.state[p]["exp_avg_sq"] / (1 - betas[1] ** t), rtol=1e-5, atol=1e-12)
+
+
+def lookahead_radam_float64(params, grads, *, lr, betas, eps, wd, k, alpha):
+    """Lookahead (Zhang et al. 2019) wrapped around RAdam (Liu et al. 2020) as the two papers state
+    them: raw moving averages, explicit bias corrections, the length of the approximated SMA and
+    its rectification term, decoupled decay; every k-th step the slow weights move a fraction
+    alpha towards the fast ones and the fast weights restart from them.  float64 throughout."""
+    b1, b2 = betas
+    rho_inf = 2 / (1 - b2) - 1
+    out = []
+    for i, p0 in enumerate(params):
+        fast = p0.double().numpy().copy()
+        slow = fast.copy()
+        m = np.zeros_like(fast); v = np.zeros_like(fast)
+        for t, gs in enumerate(grads, 1):
+            g = gs[i].double().numpy()
+            fast = fast * (1 - lr * wd)
+            m = b1 * m + (1 - b1) * g
+            v = b2 * v + (1 - b2) * g * g
+            mh = m / (1 - b1**t)
+            rho = rho_inf - 2 * t * b2**t / (1 - b2**t)
+            if rho > 5:
+                rect = math.sqrt((rho - 4) * (rho - 2) * rho_inf / ((rho_inf - 4) * (rho_inf - 2) * rho))
+                fast = fast - lr * rect * mh / (np.sqrt(v / (1 - b2**t)) + eps)
+            else:
+                fast = fast - lr * mh
+            if t % k == 0:
+                slow = slow + alpha * (fast - slow)
+                fast = slow.copy()
+        out.append((fast, slow))
+    return out
+
+
+@pytest.mark.parametrize("engine", ENGINES)
+@pytest.mark.parametrize("k,alpha", [(6, 0.5), (3, 0.8)])
+def test_ranger_matches_lookahead_over_radam(engine, k, alpha):
+    hyper = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
+    params, grads = draw(13, steps=14)
+    eng = run(engine, "ranger", params, grads, k=k, alpha=alpha, **hyper)
+    want = lookahead_radam_float64(params, grads, lr=hyper["lr"], betas=hyper["betas"], eps=hyper["eps"],
+                                   wd=hyper["weight_decay"], k=k, alpha=alpha)
+    for i, (fast, slow) in enumerate(want):
+        for what, got, w in (("param", eng.params[i], fast), ("la_param", eng.state[i]["la_param"], slow)):
+            got = got.double().numpy()
+            bad = np.abs(got - w) > 1e-6 + 1e-5 * np.abs(w)
+            assert bad.sum() == 0, f"ranger k={k} tensor {i} {what}: {bad.sum()} elements off, max {np.abs(got - w).max()}"
+    # the periodic synchronisation really happened: with k = 3 the parameters differ from plain RAdam's
+    radam = run(engine, "radam", params, grads, decouple_wd=True, **hyper)
+    assert not torch.equal(radam.params[0], eng.params[0])
 
 
 @pytest.mark.parametrize("engine", ENGINES)
