@@ -197,7 +197,7 @@ def release_bench(args):
     if args.coalesce_numel is not None:
         opt.gradient_release_coalesce = args.coalesce_numel
     if args.coalesce_window is not None:
-        opt._QUEUE_MAX_ELEMENTS = args.coalesce_window
+        opt._QUEUE_MAX_BYTES = args.coalesce_window
     optimi_amd.prepare_for_gradient_release(model, opt)
 
     def one_pass(i):
@@ -245,7 +245,7 @@ def main():
     ap.add_argument("--coalesce-numel", type=int, default=None,
                     help="gradient-release workloads: park tensors of at most this many elements (default: the optimizer's)")
     ap.add_argument("--coalesce-window", type=int, default=None,
-                    help="gradient-release workloads: launch when this many elements are parked (default: the optimizer's)")
+                    help="gradient-release workloads: launch when this many bytes of gradients are parked (default: the optimizer's)")
     args = ap.parse_args()
 
     if args.gpus != 1:

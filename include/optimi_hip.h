@@ -45,8 +45,13 @@ enum optimi_flags {
   OPTIMI_DECOUPLE_LR = 16,/* StableAdamW: fully decoupled decay (optimi/stableadamw.py:453-457)   */
   OPTIMI_DAMPENING = 32,  /* SGD: momentum buffer is an EMA, lerp(m, g, 1-momentum) (optimi/sgd.py:352-353) */
   OPTIMI_RECTIFY = 64,    /* RAdam/Ranger: rho > 5, take the rectified Adam step (optimi/radam.py:269-277) */
-  OPTIMI_LOOKAHEAD = 128  /* Ranger: this step synchronises with the slow weights, step % k == 0
+  OPTIMI_LOOKAHEAD = 128, /* Ranger: this step synchronises with the slow weights, step % k == 0
                              (optimi/ranger.py:452, 471)                                           */
+  OPTIMI_COLD = 256       /* whole-list entry points: the tensors were not touched recently (they are a
+                             slice of a larger model, e.g. small tensors gathered during gradient
+                             release).  A hint: a short list otherwise counts as resident in the
+                             last-level cache and is read with cached instead of streaming loads.
+                             Results do not depend on it.  No counterpart in the reference.        */
 };
 
 enum optimi_status {
@@ -75,7 +80,8 @@ int64_t optimi_hip_chunk_elems(int dtype);
  * the device-side tensor table (pointers, sizes), the chunk map, StableAdamW's
  * reduction partials and per-tensor scalars, and a small pinned staging ring.  None
  * of it is optimizer state; it can be dropped and rebuilt at any time.  Tables are
- * re-uploaded only when a pointer or size differs from the previous call.  A group
+ * re-uploaded only when a pointer or size differs from the previous call; a list of at most
+ * 16 tensors needs no tables at all (its pointers travel as kernel arguments).  A group
  * belongs to the device that was current when it was created and must be used by
  * one thread and one stream at a time.  (No counterpart in the reference: it plays
  * the role of the Python loop in optimi/adam.py:551-583.)

@@ -31,8 +31,17 @@
 #include <vector>
 
 #include "optimi_hip.h"
+#include "tables.h"
 
 namespace {
+
+using optimi_tables::bit;
+using optimi_tables::FewTable;
+using optimi_tables::kChunkBytes;
+using optimi_tables::kFew;
+using optimi_tables::kMaxArrays;
+using optimi_tables::TensorEntry;
+using optimi_tables::valid_dtype;
 
 #ifndef OPTIMI_THREADS
 #define OPTIMI_THREADS 64
@@ -42,13 +51,11 @@ namespace {
 #endif
 constexpr int kThreads = OPTIMI_THREADS;  // lanes per workgroup
 constexpr int kUnroll = OPTIMI_UNROLL;    // 16-byte vectors per lane per array
-constexpr int kChunkBytes = 16384;        // bytes per array per chunk: the granule of the chunk map
 constexpr int kSub = kChunkBytes / (kThreads * kUnroll * 16);  // workgroups per chunk
 static_assert(kSub >= 1 && kSub * kThreads * kUnroll * 16 == kChunkBytes, "workgroup tile must divide the chunk");
 static_assert(kThreads % 64 == 0 && kThreads <= 1024, "whole wavefronts");
 constexpr int kReduceThreads = 1024;      // lanes of the per-tensor finalize workgroup
-constexpr int kMaxArrays = 7;   // Adan: p g m diff sq prev kahan
-constexpr int kAbiVersion = 1000;
+constexpr int kAbiVersion = 1001;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -58,15 +65,12 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 // Pointers come out of the tensor table as plain addresses; telling the compiler they are
 // global memory gets global_load/global_store instead of flat accesses.
 #define OPTIMI_GLOBAL __attribute__((address_space(1)))
-#ifndef OPTIMI_LOAD_NT
-#define OPTIMI_LOAD_NT 1  // 16-byte loads carry the `nt` policy (tuning builds set 0 to compare)
-#endif
-__device__ __forceinline__ u32x4 load16(const void* base, int64_t byte_off) {
-#if OPTIMI_LOAD_NT
-  return __builtin_nontemporal_load((const OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
-#else
-  return *(const OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off);
-#endif
+// `streaming`: the data will not be used again before it has left every cache (`nt` policy).
+// Without it the load is an ordinary cached one, which is what a working set small enough to
+// stay in the 256 MB last-level cache between steps wants.  The flag is wave-uniform.
+__device__ __forceinline__ u32x4 load16(const void* base, int64_t byte_off, bool streaming) {
+  const OPTIMI_GLOBAL u32x4* p = (const OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off);
+  return streaming ? __builtin_nontemporal_load(p) : *p;
 }
 __device__ __forceinline__ void store16(void* base, int64_t byte_off, u32x4 v) {
   __builtin_nontemporal_store(v, (OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
@@ -175,15 +179,6 @@ struct F16 {
 // ------------------------------------------------------------------------------------
 // tables
 // ------------------------------------------------------------------------------------
-struct TensorEntry {
-  void* ptr[kMaxArrays];
-  int64_t numel;
-  int64_t first_chunk;  // index of this tensor's first chunk within the launch
-  uint32_t vec_ok;      // all buffers 16-byte aligned
-  uint32_t pad;
-};
-static_assert(sizeof(TensorEntry) == 80, "TensorEntry layout");
-
 struct TensorScalars {  // StableAdamW: what pass 2 needs per tensor, written on the device
   float neg_lr;
   float wd_factor;
@@ -208,8 +203,6 @@ __device__ __forceinline__ void kahan_commit(f32x2& p, f32x2& k) {
   f32x2 err = DT::R2(old - p);
   k = DT::R2(k + err);
 }
-
-constexpr uint32_t bit(int i) { return 1u << i; }
 
 // ------------------------------------------------------------------------------------
 // element functions on pairs.  x[] is indexed by array slot; each Op names its slots.
@@ -571,11 +564,17 @@ __device__ __forceinline__ void compute_store(const TensorEntry& e, int64_t off,
 }
 
 template <class Op>
-__device__ __forceinline__ void load_vec(const TensorEntry& e, int64_t off, u32x4* raw) {
+__device__ __forceinline__ void load_vec(const TensorEntry& e, int64_t off, u32x4* raw, bool streaming) {
   using DT = typename Op::DT;
+  if (streaming) {
 #pragma unroll
-  for (int a = 0; a < Op::kArrays; ++a)
-    if (Op::kLoad & bit(a)) raw[a] = load16(e.ptr[a], off * DT::kElemBytes);
+    for (int a = 0; a < Op::kArrays; ++a)
+      if (Op::kLoad & bit(a)) raw[a] = load16(e.ptr[a], off * DT::kElemBytes, true);
+  } else {
+#pragma unroll
+    for (int a = 0; a < Op::kArrays; ++a)
+      if (Op::kLoad & bit(a)) raw[a] = load16(e.ptr[a], off * DT::kElemBytes, false);
+  }
 }
 
 template <class Op>
@@ -593,10 +592,16 @@ __device__ __forceinline__ void one_element(const TensorEntry& e, int64_t i, con
     if (Op::kStore & bit(a)) DT::store1(e.ptr[a], i, x[a].x);
 }
 
+// Launch policy bits (kernel argument).
+constexpr uint32_t kPolicyCachedLoads = 1;  // ordinary cached loads instead of `nt` ones
+
+// MULTI: the tensor table and the chunk map are in device memory.  Otherwise the table travels
+// as the kernel argument `few` (one tensor for the per-tensor entry points, up to kFew for
+// short lists) and the workgroup searches it.
 template <class Op, bool MULTI>
 __global__ void __launch_bounds__(kThreads)
-step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, const TensorEntry single,
-            typename Op::Scalars s, double* __restrict__ partials) {
+step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, const FewTable few,
+            typename Op::Scalars s, double* __restrict__ partials, uint32_t policy) {
   using DT = typename Op::DT;
   constexpr int V = DT::kVec;
   constexpr int A = Op::kArrays;
@@ -605,12 +610,11 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
 
   const int64_t chunk_id = blockIdx.x / kSub;
   const int sub = blockIdx.x % kSub;
-  int tensor = 0;
-  if (MULTI) tensor = chunk_map[chunk_id];
-  const TensorEntry& e = MULTI ? table[tensor] : single;
-  const int64_t chunk = chunk_id - (MULTI ? e.first_chunk : 0);
-  const int64_t base = chunk * kChunk + sub * kTile;
+  const int tensor = MULTI ? chunk_map[chunk_id] : optimi_tables::few_lookup(few, chunk_id);
+  const TensorEntry& e = MULTI ? table[tensor] : few.e[tensor];
+  const int64_t base = optimi_tables::tile_base(chunk_id, sub, e.first_chunk, kChunk, kTile);
   const int64_t remain = e.numel - base;  // <= 0 for tiles past the end of the tensor's last chunk
+  const bool streaming = !(policy & kPolicyCachedLoads);
   Op::prepare(s, tensor);
 
   float acc = 0.0f;
@@ -618,7 +622,7 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
     // full tile: every load is issued before the first use
     u32x4 raw[kUnroll][A];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) load_vec<Op>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u]);
+    for (int u = 0; u < kUnroll; ++u) load_vec<Op>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u], streaming);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
       compute_store<Op, true>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u], s, acc, base);
@@ -629,7 +633,7 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
       const int64_t off = base + ((int64_t)u * kThreads + threadIdx.x) * V;
       if (off + V <= end) {
         u32x4 raw[A];
-        load_vec<Op>(e, off, raw);
+        load_vec<Op>(e, off, raw, streaming);
         compute_store<Op>(e, off, raw, s, acc);
       } else {
         for (int64_t i = off; i < end; ++i) one_element<Op>(e, i, s, acc);
@@ -659,11 +663,11 @@ struct FinalizeArgs {
 
 template <class DT, bool MULTI>
 __global__ void __launch_bounds__(kReduceThreads)
-stable_finalize_kernel(const TensorEntry* __restrict__ table, const TensorEntry single, const double* __restrict__ partials,
+stable_finalize_kernel(const TensorEntry* __restrict__ table, const FewTable few, const double* __restrict__ partials,
                        TensorScalars* __restrict__ out, FinalizeArgs a) {
   constexpr int64_t kChunk = chunk_elems<DT>();
-  const TensorEntry& e = MULTI ? table[blockIdx.x] : single;
-  const int64_t first = (MULTI ? e.first_chunk : 0) * kSub;  // one partial per workgroup of pass 1
+  const TensorEntry& e = MULTI ? table[blockIdx.x] : few.e[blockIdx.x];
+  const int64_t first = e.first_chunk * kSub;  // one partial per workgroup of pass 1
   const int64_t count = (e.numel + kChunk - 1) / kChunk * kSub;
   // four independent accumulators keep several loads in flight; the order is fixed, so the sum is
   // the same on every run
@@ -703,6 +707,7 @@ __global__ void __launch_bounds__(256) copy_probe_kernel(u32x4* __restrict__ dst
 // ------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------
+constexpr int popcount(uint32_t x) { return x ? (int)(x & 1u) + popcount(x >> 1) : 0; }
 inline float S(double x) { return (float)x; }
 inline float round_bf16_host(float f) {
   uint32_t u;
@@ -716,7 +721,6 @@ inline float round_f16_host(float f) { return (float)(_Float16)f; }  // round-to
 inline float Sd(double x, int dtype) {
   return dtype == OPTIMI_BF16 ? round_bf16_host((float)x) : dtype == OPTIMI_F16 ? round_f16_host((float)x) : (float)x;
 }
-inline bool valid_dtype(int dtype) { return dtype == OPTIMI_F32 || dtype == OPTIMI_BF16 || dtype == OPTIMI_F16; }
 inline Lerp make_lerp(double weight) {
   float w = (float)weight;
   Lerp l;
@@ -724,8 +728,8 @@ inline Lerp make_lerp(double weight) {
   l.coef = l.small ? w : w - 1.0f;
   return l;
 }
-inline int64_t chunk_elems_rt(int dtype) { return dtype == OPTIMI_F32 ? chunk_elems<F32>() : chunk_elems<BF16>(); }
-inline int elem_bytes(int dtype) { return dtype == OPTIMI_F32 ? 4 : 2; }
+inline int64_t chunk_elems_rt(int dtype) { return optimi_tables::chunk_elems(dtype); }
+using optimi_tables::elem_bytes;
 
 #define HIP_TRY(expr)                          \
   do {                                         \
@@ -769,7 +773,6 @@ struct optimi_group {
   std::vector<int32_t> host_map;         // scratch for building the chunk map
   std::vector<int64_t> map_numel;        // sizes the device chunk map was built for
   int64_t map_chunk = 0;
-  int64_t n_chunks = 0;
   StagingSlot ring[4];
   int ring_pos = 0;
   hipEvent_t last_launch = nullptr;
@@ -805,54 +808,63 @@ int staged_upload(optimi_group* g, void* dst, const void* src, size_t bytes, hip
 
 int check_ptrs(int n_tensors, const void* const* list) { return (n_tensors > 0 && list == nullptr) ? OPTIMI_ERR_NULL : 0; }
 
-// Validates the list, (re)builds the chunk map and tensor table and uploads what changed.
+// What one list launch works on, as the entry points hand it to the launchers.
+struct ListPlan {
+  bool few = false;           // the table travels as a kernel argument; the group's tables are untouched
+  FewTable table;             // valid when `few`
+  int n_tensors = 0;
+  int64_t n_chunks = 0;
+  int64_t footprint = 0;      // bytes of all arrays the launch touches
+  bool cold = false;          // the caller said the tensors were not touched recently (OPTIMI_COLD)
+};
+
+constexpr int64_t kMaxChunks = (int64_t)0x7fffffff / kSub;  // the grid is chunks x kSub workgroups
+
+// Validates the list and gets its tables to where the kernel reads them: into `plan` itself for
+// a list of at most kFew tensors (nothing is uploaded), else into the group's device tables,
+// (re)building the chunk map and tensor table and uploading what changed.
 // `lists[a]` may be nullptr for an array the launch does not touch (`need` has its bit clear).
-int prepare_tables(optimi_group* g, int n_tensors, const void* const* const* lists, int n_arrays, uint32_t need,
-                   const int64_t* numel, int dtype, hipStream_t stream) {
+int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, int n_arrays, uint32_t need,
+              const int64_t* numel, int dtype, uint32_t flags, hipStream_t stream, ListPlan* plan) {
   if (!g) return OPTIMI_ERR_NULL;
   if (n_tensors < 0) return OPTIMI_ERR_SIZE;
   if (!valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
-  if (n_tensors > 0 && !numel) return OPTIMI_ERR_NULL;
-  for (int a = 0; a < n_arrays; ++a)
-    if ((need & bit(a)) && check_ptrs(n_tensors, lists[a])) return OPTIMI_ERR_NULL;
   int dev = 0;
   HIP_TRY(hipGetDevice(&dev));
   if (dev != g->device) return OPTIMI_ERR_DEVICE;
 
   const int64_t chunk = chunk_elems_rt(dtype);
-  const int eb = elem_bytes(dtype);
+  plan->n_tensors = n_tensors;
+  plan->cold = (flags & OPTIMI_COLD) != 0;
+  plan->few = n_tensors <= kFew;
+  std::memset(&plan->table, 0, sizeof(plan->table));
   std::vector<TensorEntry> fresh;
-  try {
-    fresh.resize((size_t)n_tensors);
-  } catch (const std::bad_alloc&) {
-    return OPTIMI_ERR_NOMEM;
+  TensorEntry* entries = plan->table.e;
+  if (!plan->few) {
+    try {
+      fresh.resize((size_t)n_tensors);
+    } catch (const std::bad_alloc&) {
+      return OPTIMI_ERR_NOMEM;
+    }
+    entries = fresh.data();
   }
   int64_t n_chunks = 0;
-  for (int t = 0; t < n_tensors; ++t) {
-    TensorEntry& e = fresh[(size_t)t];
-    std::memset(&e, 0, sizeof(e));
-    if (numel[t] < 0) return OPTIMI_ERR_SIZE;
-    e.numel = numel[t];
-    e.first_chunk = n_chunks;
-    e.vec_ok = 1;
-    for (int a = 0; a < n_arrays; ++a) {
-      if (!(need & bit(a))) continue;
-      const void* p = lists[a][t];
-      if (!p && numel[t] > 0) return OPTIMI_ERR_NULL;
-      uintptr_t u = (uintptr_t)p;
-      if (u % (uintptr_t)eb) return OPTIMI_ERR_ALIGN;
-      if (u % 16) e.vec_ok = 0;
-      e.ptr[a] = const_cast<void*>(p);
-    }
-    n_chunks += (numel[t] + chunk - 1) / chunk;
+  int rc = optimi_tables::build_entries(n_tensors, lists, n_arrays, need, numel, dtype, kMaxChunks, entries, &n_chunks);
+  if (rc) return rc;
+  plan->n_chunks = n_chunks;
+  int64_t total = 0;
+  for (int t = 0; t < n_tensors; ++t) total += numel[t];
+  plan->footprint = total * elem_bytes(dtype) * popcount(need);
+  if (plan->few) {
+    plan->table.n = n_tensors;
+    return 0;
   }
-  if (n_chunks * kSub > 0x7fffffff) return OPTIMI_ERR_SIZE;
 
   // a group moved to another stream must not overwrite tables a previous launch still reads
   if (g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
 
   bool same_sizes = g->map_chunk == chunk && g->map_numel.size() == (size_t)n_tensors &&
-                    (n_tensors == 0 || std::memcmp(g->map_numel.data(), numel, sizeof(int64_t) * (size_t)n_tensors) == 0);
+                    std::memcmp(g->map_numel.data(), numel, sizeof(int64_t) * (size_t)n_tensors) == 0;
   if (!same_sizes && n_chunks > 0) {
     g->map_chunk = 0;  // the cached map is void until the new one is on its way
     try {
@@ -861,23 +873,18 @@ int prepare_tables(optimi_group* g, int n_tensors, const void* const* const* lis
     } catch (const std::bad_alloc&) {
       return OPTIMI_ERR_NOMEM;
     }
-    for (int t = 0; t < n_tensors; ++t) {
-      const int64_t c0 = fresh[(size_t)t].first_chunk;
-      const int64_t c1 = c0 + (numel[t] + chunk - 1) / chunk;
-      for (int64_t c = c0; c < c1; ++c) g->host_map[(size_t)c] = t;
-    }
-    int rc = g->chunk_map.reserve(sizeof(int32_t) * (size_t)n_chunks);
+    optimi_tables::build_chunk_map(fresh.data(), n_tensors, chunk, g->host_map.data());
+    rc = g->chunk_map.reserve(sizeof(int32_t) * (size_t)n_chunks);
     if (rc) return rc;
     rc = staged_upload(g, g->chunk_map.ptr, g->host_map.data(), sizeof(int32_t) * (size_t)n_chunks, stream);
     if (rc) return rc;
     g->map_chunk = chunk;
   }
-  g->n_chunks = n_chunks;
 
   bool same_table = g->host_table.size() == fresh.size() &&
-                    (fresh.empty() || std::memcmp(g->host_table.data(), fresh.data(), sizeof(TensorEntry) * fresh.size()) == 0);
-  if (!same_table && n_tensors > 0) {
-    int rc = g->table.reserve(sizeof(TensorEntry) * fresh.size());
+                    std::memcmp(g->host_table.data(), fresh.data(), sizeof(TensorEntry) * fresh.size()) == 0;
+  if (!same_table) {
+    rc = g->table.reserve(sizeof(TensorEntry) * fresh.size());
     if (rc) {
       g->host_table.clear();
       return rc;
@@ -901,19 +908,44 @@ int note_launch(optimi_group* g, hipStream_t stream) {
   return 0;
 }
 
+// After a list launch: a launch that used the group's device tables is recorded so that the
+// next use of the group on another stream waits for it; a short list touched nothing of the group.
+int finish_list(optimi_group* g, const ListPlan& plan, hipStream_t stream) {
+  if (!plan.few) return note_launch(g, stream);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 // Occupancy throttle.  HBM serves this read-modify-write mix best when a CU keeps only a
 // certain number of wavefronts resident - fewer the more 16-byte-per-lane streams (loads plus
 // stores) each wavefront carries; beyond it the achieved bandwidth drops by several per cent,
-// below it the CU cannot cover the latency.  The table is the measured optimum on MI355X with
-// the write-through tile stores (7B-parameter lists; 5 streams = StableAdamW pass 1, 6 = pass
-// 2, 7 = Lion / SGD, 9 = Adam with Kahan, 13 = Adan; entries in between are interpolated).
-// fp32 lists with 7 streams do best one wavefront above the 16-bit ones.  The cap is imposed
-// with a dynamic-LDS request that no kernel touches: a CU has 160 KiB of LDS, so asking for L
-// bytes leaves room for floor(160 KiB / L) workgroups.  OPTIMI_HIP_WAVES overrides the number
-// of wavefronts per CU for every kernel (0 = no throttle); it is read once.
-constexpr int kLdsPerCu = 160 * 1024;
+// below it the CU cannot cover the latency.  The cap is imposed with a dynamic-LDS request that
+// no kernel touches.  A CU hands its 160 KiB of LDS out in 128 granules of 1280 bytes (measured:
+// swept over the request size, the achieved bandwidth moves in steps exactly where the granule
+// count changes), so a workgroup that asks for g granules leaves room for floor(128 / g)
+// workgroups; reachable occupancies are therefore 32, 25, 21, 18, 16, 14, 12, 11, 10, 9, 8, ...
+// The table holds the measured optimum in granules on MI355X with the write-through tile stores
+// (7B-parameter lists; 5 streams = StableAdamW pass 1 and accumulate-only Adam, 6 = pass 2,
+// 7 = Lion / SGD, 9 = Adam with Kahan, 13 = Adan; entries in between are interpolated).  fp32
+// lists with 7 streams do best at 12 workgroups instead of 11.  16-bit launches of fewer than
+// kLongLaunch workgroups (the Llama-1B-shaped list, single tensors) do best one granule lower,
+// i.e. with one more workgroup resident.  OPTIMI_HIP_WAVES overrides the number of wavefronts
+// per CU for every kernel (nearest reachable count at or above it; 0 = no throttle); read once.
+constexpr int kLdsGranule = 1280, kLdsGranules = 128;
 constexpr int kMaxStreams = 2 * kMaxArrays;
-constexpr int kBestWaves[kMaxStreams + 1] = {32, 32, 32, 32, 24, 17, 17, 12, 12, 11, 10, 9, 8, 8, 8};
+constexpr int kBestGranules[kMaxStreams + 1] = {4, 4, 4, 4, 6, 8, 8, 11, 11, 12, 13, 14, 16, 16, 16};
+constexpr int64_t kLongLaunch = (int64_t)1 << 22;  // workgroups
+
+// A list whose arrays add up to at most this many bytes stays in the 256 MB last-level cache
+// from one optimizer step to the next (measured: cached loads beat `nt` loads up to 270 MB of
+// arrays and lose from 335 MB on).  Such a launch - unless the caller marks it OPTIMI_COLD -
+// uses cached loads and, being short, 21 resident workgroups per CU (16.8 M fp32 parameters in
+// one launch: 83 us -> 78 us).  Per-tensor entry points never take this path: they step one
+// tensor of a larger model, which was last touched a whole backward pass ago (measured on
+// tensors that are cold when revisited: `nt` loads and the table's occupancy are 6-8 % faster
+// there than cached loads or 21 workgroups).
+constexpr int64_t kResidentBytes = (int64_t)288 << 20;
+constexpr int kResidentGranules = 6;
 
 int forced_waves() {
 #ifdef OPTIMI_TUNING
@@ -927,47 +959,74 @@ int forced_waves() {
   return value;
 }
 
-constexpr int popcount(uint32_t x) { return x ? (int)(x & 1u) + popcount(x >> 1) : 0; }
-
-// A short launch - fewer than kShortRounds rounds of resident workgroups over the 256 CUs - is
-// dominated by filling and draining the chip, not by the steady state the table is tuned for,
-// and does better with more wavefronts in flight (16.8 M fp32 parameters in one launch: 102 us
-// at 13 per CU, 96 us at 20).
-constexpr int kShortRounds = 24, kShortWaves = 20, kCus = 256;
+struct LaunchShape {
+  unsigned lds;     // dynamic LDS request in bytes (the occupancy throttle)
+  uint32_t policy;  // kPolicy* bits
+};
 
 template <class Op>
-unsigned throttle_lds(int64_t workgroups) {
+LaunchShape launch_shape(int64_t workgroups, bool resident) {
   constexpr int streams = (popcount(Op::kLoad) + popcount(Op::kStore)) * kUnroll;
   constexpr bool f32 = std::is_same<typename Op::DT, F32>::value;
-  int waves = kBestWaves[streams < kMaxStreams ? streams : kMaxStreams] + ((f32 && streams == 7) ? 1 : 0);
-  if (workgroups * (kThreads / 64) < (int64_t)kShortRounds * kCus * waves && waves < kShortWaves) waves = kShortWaves;
+  LaunchShape shape;
+  shape.policy = resident ? kPolicyCachedLoads : 0u;
+  int granules = kBestGranules[streams < kMaxStreams ? streams : kMaxStreams];
+  if (f32 && streams == 7) granules = 10;
+  if (!f32 && streams >= 7 && workgroups < kLongLaunch) granules -= 1;
+  if (resident) granules = kResidentGranules;
 #ifdef OPTIMI_TUNING
-  if (const char* env = std::getenv("OPTIMI_HIP_LDS")) return (unsigned)std::strtol(env, nullptr, 10);  // raw request, tuning builds only
+  if (const char* env = std::getenv("OPTIMI_HIP_LDS")) {  // raw request, tuning builds only
+    shape.lds = (unsigned)std::strtol(env, nullptr, 10);
+    return shape;
+  }
 #endif
   const int forced = forced_waves();
-  if (forced == 0) return 0;
-  if (forced > 0) waves = forced;
-  int wgs = waves / (kThreads / 64);
-  if (wgs < 1) wgs = 1;
-  // midway between "wgs fit" and "wgs + 1 fit", so allocation granularity cannot tip it
-  long lds = (long)(2L * kLdsPerCu / (2 * wgs + 1));
-  if (lds > 65536) lds = 65536;
-  return (unsigned)lds;
+  if (forced == 0) {
+    shape.lds = 0;
+    return shape;
+  }
+  if (forced > 0) {
+    const int wgs = forced / (kThreads / 64) > 0 ? forced / (kThreads / 64) : 1;
+    granules = kLdsGranules / wgs;
+  }
+  if (granules < 1) granules = 1;
+  if (granules > 51) granules = 51;  // a workgroup may ask for 64 KiB at most
+  // a little under the granule boundary: the kernel's own static LDS (a few bytes in the
+  // reducing kernels) is added to the request and must not tip it into the next granule
+  shape.lds = (unsigned)(granules * kLdsGranule - 128);
+  return shape;
 }
 
+const FewTable kNoTable = {};
+
 template <class Op>
-void launch_multi(optimi_group* g, const typename Op::Scalars& s, hipStream_t stream, double* partials = nullptr) {
-  TensorEntry none;
-  std::memset(&none, 0, sizeof(none));
-  step_kernel<Op, true><<<dim3((unsigned)(g->n_chunks * kSub)), dim3(kThreads), throttle_lds<Op>(g->n_chunks * kSub), stream>>>(
-      (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, none, s, partials);
+void launch_list(optimi_group* g, const ListPlan& plan, const typename Op::Scalars& s, hipStream_t stream,
+                 double* partials = nullptr) {
+  const int64_t workgroups = plan.n_chunks * kSub;
+  const LaunchShape shape = launch_shape<Op>(workgroups, !plan.cold && plan.footprint <= kResidentBytes);
+  if (plan.few)
+    step_kernel<Op, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
+        nullptr, nullptr, plan.table, s, partials, shape.policy);
+  else
+    step_kernel<Op, true><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
+        (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, partials, shape.policy);
+}
+
+inline FewTable table_of_one(const TensorEntry& e) {
+  FewTable one = {};
+  one.e[0] = e;
+  one.e[0].first_chunk = 0;
+  one.n = 1;
+  return one;
 }
 
 template <class Op>
 void launch_single(const TensorEntry& e, const typename Op::Scalars& s, double* partials, hipStream_t stream) {
   const int64_t chunk = chunk_elems<typename Op::DT>();
-  const unsigned blocks = (unsigned)((e.numel + chunk - 1) / chunk * kSub);
-  step_kernel<Op, false><<<dim3(blocks), dim3(kThreads), throttle_lds<Op>(blocks), stream>>>(nullptr, nullptr, e, s, partials);
+  const int64_t workgroups = (e.numel + chunk - 1) / chunk * kSub;
+  const LaunchShape shape = launch_shape<Op>(workgroups, false);
+  step_kernel<Op, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
+      nullptr, nullptr, table_of_one(e), s, partials, shape.policy);
 }
 
 // Calls fn(Op{}) for the Op selected by dtype x kahan x update x weight-decay mode.  NWD is
@@ -1167,15 +1226,16 @@ int64_t stable_partials(int64_t numel) {  // pass-1 workgroups of one tensor
 
 // `scratch` is written before it is read within the call (every pass-1 workgroup stores its
 // partial, finalize stores the scalars), so it needs no clearing between calls.
+// `plan`: the list to step, or nullptr to step the one tensor `single`.
 template <class DT>
-int stable_run(bool multi, optimi_group* g, const TensorEntry& single, int n_tensors, const StableScratch& scratch,
+int stable_run(const ListPlan* plan, optimi_group* g, const TensorEntry& single, const StableScratch& scratch,
                int dtype, double lr, double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay,
                double eps, double max_lr, uint32_t flags, hipStream_t stream) {
   const bool update = (flags & OPTIMI_UPDATE) != 0;
   const bool kahan = kahan_on(dtype, flags);
   StableP1Scalars s1 = stable_p1_scalars(dtype, beta1_comp, beta2_hat, beta2_comp, eps);
   if (!update) {
-    if (multi) launch_multi<StablePass1Op<DT, false>>(g, s1, stream);
+    if (plan) launch_list<StablePass1Op<DT, false>>(g, *plan, s1, stream);
     else launch_single<StablePass1Op<DT, false>>(single, s1, nullptr, stream);
     return 0;
   }
@@ -1190,20 +1250,22 @@ int stable_run(bool multi, optimi_group* g, const TensorEntry& single, int n_ten
   s2.neg_lr = 0.0f;
   s2.wd = 0.0f;
   const bool wd = weight_decay != 0;
-  if (multi) {
-    launch_multi<StablePass1Op<DT, true>>(g, s1, stream, scratch.partials);
-    TensorEntry none;
-    std::memset(&none, 0, sizeof(none));
-    stable_finalize_kernel<DT, true><<<dim3((unsigned)n_tensors), dim3(kReduceThreads), 0, stream>>>(
-        (const TensorEntry*)g->table.ptr, none, scratch.partials, scratch.tensor_scalars, fa);
-    if (kahan && wd) launch_multi<StablePass2Op<DT, true, 1>>(g, s2, stream);
-    else if (kahan) launch_multi<StablePass2Op<DT, true, 0>>(g, s2, stream);
-    else if (wd) launch_multi<StablePass2Op<DT, false, 1>>(g, s2, stream);
-    else launch_multi<StablePass2Op<DT, false, 0>>(g, s2, stream);
+  if (plan) {
+    launch_list<StablePass1Op<DT, true>>(g, *plan, s1, stream, scratch.partials);
+    if (plan->few)
+      stable_finalize_kernel<DT, false><<<dim3((unsigned)plan->n_tensors), dim3(kReduceThreads), 0, stream>>>(
+          nullptr, plan->table, scratch.partials, scratch.tensor_scalars, fa);
+    else
+      stable_finalize_kernel<DT, true><<<dim3((unsigned)plan->n_tensors), dim3(kReduceThreads), 0, stream>>>(
+          (const TensorEntry*)g->table.ptr, kNoTable, scratch.partials, scratch.tensor_scalars, fa);
+    if (kahan && wd) launch_list<StablePass2Op<DT, true, 1>>(g, *plan, s2, stream);
+    else if (kahan) launch_list<StablePass2Op<DT, true, 0>>(g, *plan, s2, stream);
+    else if (wd) launch_list<StablePass2Op<DT, false, 1>>(g, *plan, s2, stream);
+    else launch_list<StablePass2Op<DT, false, 0>>(g, *plan, s2, stream);
   } else {
     launch_single<StablePass1Op<DT, true>>(single, s1, scratch.partials, stream);
     stable_finalize_kernel<DT, false><<<dim3(1), dim3(kReduceThreads), 0, stream>>>(
-        nullptr, single, scratch.partials, scratch.tensor_scalars, fa);
+        nullptr, table_of_one(single), scratch.partials, scratch.tensor_scalars, fa);
     if (kahan && wd) launch_single<StablePass2Op<DT, true, 1>>(single, s2, nullptr, stream);
     else if (kahan) launch_single<StablePass2Op<DT, true, 0>>(single, s2, nullptr, stream);
     else if (wd) launch_single<StablePass2Op<DT, false, 1>>(single, s2, nullptr, stream);
@@ -1212,16 +1274,16 @@ int stable_run(bool multi, optimi_group* g, const TensorEntry& single, int n_ten
   return 0;
 }
 
-// The group's own scratch, grown to what this step needs (whole list: `multi`; else one tensor).
+// The group's own scratch, grown to what this step needs (a whole list, or one tensor).
 template <class DT>
-int group_scratch(optimi_group* g, bool multi, int64_t single_numel, int n_tensors, uint32_t flags, StableScratch* out) {
+int group_scratch(optimi_group* g, const ListPlan* plan, int64_t single_numel, uint32_t flags, StableScratch* out) {
   out->partials = nullptr;
   out->tensor_scalars = nullptr;
   if (!(flags & OPTIMI_UPDATE)) return 0;  // the accumulate-only step reduces nothing
-  const int64_t n_partials = multi ? g->n_chunks * kSub : stable_partials<DT>(single_numel);
+  const int64_t n_partials = plan ? plan->n_chunks * kSub : stable_partials<DT>(single_numel);
   int rc = g->partials.reserve(sizeof(double) * (size_t)n_partials);
   if (rc) return rc;
-  rc = g->tensor_scalars.reserve(sizeof(TensorScalars) * (size_t)(multi ? n_tensors : 1));
+  rc = g->tensor_scalars.reserve(sizeof(TensorScalars) * (size_t)(plan ? plan->n_tensors : 1));
   if (rc) return rc;
   out->partials = (double*)g->partials.ptr;
   out->tensor_scalars = (TensorScalars*)g->tensor_scalars.ptr;
@@ -1229,14 +1291,14 @@ int group_scratch(optimi_group* g, bool multi, int64_t single_numel, int n_tenso
 }
 
 template <class DT>
-int stable_group_run(bool multi, optimi_group* g, const TensorEntry& single, int n_tensors, int dtype, double lr,
+int stable_group_run(const ListPlan* plan, optimi_group* g, const TensorEntry& single, int dtype, double lr,
                      double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay, double eps,
                      double max_lr, uint32_t flags, hipStream_t stream) {
   StableScratch scratch;
-  int rc = group_scratch<DT>(g, multi, single.numel, n_tensors, flags, &scratch);
+  int rc = group_scratch<DT>(g, plan, single.numel, flags, &scratch);
   if (rc) return rc;
-  return stable_run<DT>(multi, g, single, n_tensors, scratch, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay,
-                        eps, max_lr, flags, stream);
+  return stable_run<DT>(plan, g, single, scratch, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr,
+                        flags, stream);
 }
 
 // ---- fixed scratch of the allocation-free entry point ---------------------------------------
@@ -1343,12 +1405,13 @@ int optimi_hip_adam_multi(optimi_group* g, int n_tensors, void* const* param, co
   const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
   const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
                                  (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
-  int rc = prepare_tables(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, stream);
+  ListPlan plan;
+  int rc = plan_list(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, flags, stream, &plan);
   if (rc) return rc;
-  if (g->n_chunks == 0) return 0;
+  if (plan.n_chunks == 0) return 0;
   AdamScalars s = adam_scalars(dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
-  dispatch<AdamOp, 3>(dtype, kahan, update, adam_wd_mode(weight_decay, flags), [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
-  return note_launch(g, stream);
+  dispatch<AdamOp, 3>(dtype, kahan, update, adam_wd_mode(weight_decay, flags), [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
+  return finish_list(g, plan, stream);
 }
 
 int optimi_hip_lion_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
@@ -1359,12 +1422,13 @@ int optimi_hip_lion_multi(optimi_group* g, int n_tensors, void* const* param, co
   const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
   const void* const* lists[4] = {(const void* const*)param, grad, (const void* const*)exp_avg,
                                  (const void* const*)kahan_comp};
-  int rc = prepare_tables(g, n_tensors, lists, 4, lion_need(kahan, update), numel, dtype, stream);
+  ListPlan plan;
+  int rc = plan_list(g, n_tensors, lists, 4, lion_need(kahan, update), numel, dtype, flags, stream, &plan);
   if (rc) return rc;
-  if (g->n_chunks == 0) return 0;
+  if (plan.n_chunks == 0) return 0;
   LionScalars s = lion_scalars(dtype, lr, beta1_comp, beta2_comp, weight_decay);
-  dispatch<LionOp, 2>(dtype, kahan, update, lion_wd_mode(weight_decay, flags), [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
-  return note_launch(g, stream);
+  dispatch<LionOp, 2>(dtype, kahan, update, lion_wd_mode(weight_decay, flags), [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
+  return finish_list(g, plan, stream);
 }
 
 int optimi_hip_stableadamw_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
@@ -1377,16 +1441,19 @@ int optimi_hip_stableadamw_multi(optimi_group* g, int n_tensors, void* const* pa
   const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
   const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
                                  (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
-  int rc = prepare_tables(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, stream);
+  ListPlan plan;
+  int rc = plan_list(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, flags, stream, &plan);
   if (rc) return rc;
-  if (g->n_chunks == 0) return 0;
+  if (plan.n_chunks == 0) return 0;
+  // the reduction scratch is the group's: a previous launch on another stream may still read it
+  if (plan.few && g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
   TensorEntry none;
   std::memset(&none, 0, sizeof(none));
   rc = dtype == OPTIMI_BF16
-           ? stable_group_run<BF16>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           ? stable_group_run<BF16>(&plan, g, none, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
        : dtype == OPTIMI_F16
-           ? stable_group_run<F16>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
-           : stable_group_run<F32>(true, g, none, n_tensors, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
+           ? stable_group_run<F16>(&plan, g, none, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           : stable_group_run<F32>(&plan, g, none, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
   if (rc) return rc;
   return note_launch(g, stream);
 }
@@ -1401,12 +1468,13 @@ int optimi_hip_adan_multi(optimi_group* g, int n_tensors, void* const* param, co
   const void* const* lists[7] = {(const void* const*)param, grad, (const void* const*)exp_avg,
                                  (const void* const*)exp_avg_diff, (const void* const*)exp_avg_sq,
                                  (const void* const*)prev_grad, (const void* const*)kahan_comp};
-  int rc = prepare_tables(g, n_tensors, lists, 7, adan_need(kahan, update), numel, dtype, stream);
+  ListPlan plan;
+  int rc = plan_list(g, n_tensors, lists, 7, adan_need(kahan, update), numel, dtype, flags, stream, &plan);
   if (rc) return rc;
-  if (g->n_chunks == 0) return 0;
+  if (plan.n_chunks == 0) return 0;
   AdanScalars s = adan_scalars(dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay);
-  dispatch<AdanOp, 3>(dtype, kahan, update, adan_wd_mode(weight_decay, flags), [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
-  return note_launch(g, stream);
+  dispatch<AdanOp, 3>(dtype, kahan, update, adan_wd_mode(weight_decay, flags), [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
+  return finish_list(g, plan, stream);
 }
 
 int optimi_hip_adam_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* kahan_comp,
@@ -1459,10 +1527,10 @@ int optimi_hip_stableadamw_single(optimi_group* g, void* param, const void* grad
   if (dev != g->device) return OPTIMI_ERR_DEVICE;
   if (g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
   rc = dtype == OPTIMI_BF16
-           ? stable_group_run<BF16>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           ? stable_group_run<BF16>(nullptr, g, e, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
        : dtype == OPTIMI_F16
-           ? stable_group_run<F16>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
-           : stable_group_run<F32>(false, g, e, 1, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
+           ? stable_group_run<F16>(nullptr, g, e, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           : stable_group_run<F32>(nullptr, g, e, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
   if (rc) return rc;
   return note_launch(g, stream);
 }
@@ -1489,10 +1557,10 @@ int optimi_hip_stableadamw_single_noalloc(void* param, const void* grad, void* e
   const int64_t n_partials = dtype == OPTIMI_F32 ? stable_partials<F32>(numel) : stable_partials<BF16>(numel);
   if (n_partials > kScratchPartials) return OPTIMI_ERR_LIMIT;  // the macro and the layout must agree
   rc = dtype == OPTIMI_BF16
-           ? stable_run<BF16>(false, nullptr, e, 1, sc, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           ? stable_run<BF16>(nullptr, nullptr, e, sc, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
        : dtype == OPTIMI_F16
-           ? stable_run<F16>(false, nullptr, e, 1, sc, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
-           : stable_run<F32>(false, nullptr, e, 1, sc, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
+           ? stable_run<F16>(nullptr, nullptr, e, sc, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           : stable_run<F32>(nullptr, nullptr, e, sc, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
   if (rc) return rc;
   HIP_TRY(hipGetLastError());
   return 0;
@@ -1523,12 +1591,13 @@ int optimi_hip_sgd_multi(optimi_group* g, int n_tensors, void* const* param, con
   const int mom = sgd_mom_mode(momentum, flags);
   if (!update && !mom) return g ? 0 : OPTIMI_ERR_NULL;  // nothing to accumulate into
   const void* const* lists[4] = {(const void* const*)param, grad, (const void* const*)exp_avg, (const void* const*)kahan_comp};
-  int rc = prepare_tables(g, n_tensors, lists, 4, sgd_need(kahan, update, mom), numel, dtype, stream);
+  ListPlan plan;
+  int rc = plan_list(g, n_tensors, lists, 4, sgd_need(kahan, update, mom), numel, dtype, flags, stream, &plan);
   if (rc) return rc;
-  if (g->n_chunks == 0) return 0;
+  if (plan.n_chunks == 0) return 0;
   SgdScalars s = sgd_scalars(dtype, lr, momentum, weight_decay);
-  sgd_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), mom, [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
-  return note_launch(g, stream);
+  sgd_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), mom, [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
+  return finish_list(g, plan, stream);
 }
 
 int optimi_hip_sgd_single(void* param, const void* grad, void* exp_avg, void* kahan_comp, int64_t numel, int dtype,
@@ -1557,14 +1626,15 @@ int optimi_hip_radam_multi(optimi_group* g, int n_tensors, void* const* param, c
   const bool rectify = (flags & OPTIMI_RECTIFY) != 0;
   const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
                                  (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
-  int rc = prepare_tables(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, stream);
+  ListPlan plan;
+  int rc = plan_list(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, flags, stream, &plan);
   if (rc) return rc;
-  if (g->n_chunks == 0) return 0;
+  if (plan.n_chunks == 0) return 0;
   AdamScalars s = adam_scalars(dtype, rectify ? lr * rect : lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
   const int wd = adam_wd_mode(weight_decay, flags);
-  if (rectify || !update) dispatch<AdamOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
-  else dispatch<RAdamEarlyOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
-  return note_launch(g, stream);
+  if (rectify || !update) dispatch<AdamOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
+  else dispatch<RAdamEarlyOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
+  return finish_list(g, plan, stream);
 }
 
 int optimi_hip_radam_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* kahan_comp,
@@ -1598,15 +1668,16 @@ int optimi_hip_ranger_multi(optimi_group* g, int n_tensors, void* const* param, 
   const void* const* lists[6] = {(const void* const*)param, grad, (const void* const*)exp_avg,
                                  (const void* const*)exp_avg_sq, (const void* const*)kahan_comp,
                                  (const void* const*)la_param};
-  int rc = prepare_tables(g, n_tensors, lists, 6, ranger_need(kahan, update, la), numel, dtype, stream);
+  ListPlan plan;
+  int rc = plan_list(g, n_tensors, lists, 6, ranger_need(kahan, update, la), numel, dtype, flags, stream, &plan);
   if (rc) return rc;
-  if (g->n_chunks == 0) return 0;
+  if (plan.n_chunks == 0) return 0;
   RangerScalars s;
   s.a = adam_scalars(dtype, rectify ? lr * rect : lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
   s.alpha_d = Sd(alpha, dtype);
   ranger_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), rectify, la,
-                  [&](auto op) { launch_multi<decltype(op)>(g, s, stream); });
-  return note_launch(g, stream);
+                  [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
+  return finish_list(g, plan, stream);
 }
 
 int optimi_hip_ranger_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* la_param,

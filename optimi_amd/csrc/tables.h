@@ -1,0 +1,119 @@
+// Host-side tables of a list launch: argument validation, the tensor table, the chunk map, and
+// the index arithmetic a workgroup uses to find its tile.  Plain C++ with no HIP call, so that
+// a CPU build (with sanitizers) can exercise exactly the code the library runs; the functions
+// the kernels share are marked OPTIMI_HD.
+//
+// A list of tensors is cut into chunks of kChunkBytes per array; chunks are numbered through
+// the whole list, tensor after tensor, and kSub workgroups share a chunk.  A workgroup learns
+// which tensor its chunk belongs to either from a chunk map in device memory (large lists) or,
+// for lists of at most kFew tensors, by searching a table that travels as a kernel argument.
+// This takes the place of the per-tensor Python launch loops of the reference
+// (optimi/adam.py:551-583, lion.py:470-492, stableadamw.py:689-725, adan.py:679-711).
+
+#ifndef OPTIMI_TABLES_H
+#define OPTIMI_TABLES_H
+
+#include <cstdint>
+#include <cstring>
+
+#include "optimi_hip.h"
+
+#if defined(__HIPCC__)
+#define OPTIMI_HD __host__ __device__ __forceinline__
+#else
+#define OPTIMI_HD inline
+#endif
+
+namespace optimi_tables {
+
+constexpr int kMaxArrays = 7;       // Adan: p g m diff sq prev kahan
+constexpr int kChunkBytes = 16384;  // bytes per array per chunk: the granule of the chunk map
+constexpr int kFew = 16;            // lists up to this long travel as a kernel argument
+
+struct TensorEntry {
+  void* ptr[kMaxArrays];
+  int64_t numel;
+  int64_t first_chunk;  // index of this tensor's first chunk within the launch
+  uint32_t vec_ok;      // all buffers 16-byte aligned
+  uint32_t pad;
+};
+static_assert(sizeof(TensorEntry) == 80, "TensorEntry layout");
+
+struct FewTable {
+  TensorEntry e[kFew];
+  int32_t n;
+  int32_t pad;
+};
+
+constexpr uint32_t bit(int i) { return 1u << i; }
+
+inline bool valid_dtype(int dtype) { return dtype == OPTIMI_F32 || dtype == OPTIMI_BF16 || dtype == OPTIMI_F16; }
+inline int elem_bytes(int dtype) { return dtype == OPTIMI_F32 ? 4 : 2; }
+inline int64_t chunk_elems(int dtype) { return kChunkBytes / elem_bytes(dtype); }
+inline int64_t chunks_of(int64_t numel, int64_t chunk) { return (numel + chunk - 1) / chunk; }
+
+// Validates a list and writes one entry per tensor.  `lists[a]` may be nullptr for an array the
+// launch does not touch (`need` has its bit clear).  `max_chunks` bounds the launch (the grid
+// is chunks x workgroups per chunk and must fit 31 bits).  Returns an optimi_status.
+inline int build_entries(int n_tensors, const void* const* const* lists, int n_arrays, uint32_t need, const int64_t* numel,
+                         int dtype, int64_t max_chunks, TensorEntry* out, int64_t* n_chunks_out) {
+  if (n_tensors < 0) return OPTIMI_ERR_SIZE;
+  if (!valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
+  if (n_arrays < 0 || n_arrays > kMaxArrays) return OPTIMI_ERR_SIZE;
+  if (n_tensors > 0 && (!numel || !out)) return OPTIMI_ERR_NULL;
+  for (int a = 0; a < n_arrays; ++a)
+    if ((need & bit(a)) && n_tensors > 0 && (!lists || !lists[a])) return OPTIMI_ERR_NULL;
+  const int64_t chunk = chunk_elems(dtype);
+  const uintptr_t eb = (uintptr_t)elem_bytes(dtype);
+  int64_t n_chunks = 0;
+  for (int t = 0; t < n_tensors; ++t) {
+    TensorEntry& e = out[t];
+    std::memset(&e, 0, sizeof(e));
+    if (numel[t] < 0) return OPTIMI_ERR_SIZE;
+    if (numel[t] > max_chunks * chunk) return OPTIMI_ERR_SIZE;  // also keeps the sums below from overflowing
+    e.numel = numel[t];
+    e.first_chunk = n_chunks;
+    e.vec_ok = 1;
+    for (int a = 0; a < n_arrays; ++a) {
+      if (!(need & bit(a))) continue;
+      const void* p = lists[a][t];
+      if (!p && numel[t] > 0) return OPTIMI_ERR_NULL;
+      const uintptr_t u = (uintptr_t)p;
+      if (u % eb) return OPTIMI_ERR_ALIGN;
+      if (u % 16) e.vec_ok = 0;
+      e.ptr[a] = const_cast<void*>(p);
+    }
+    n_chunks += chunks_of(numel[t], chunk);
+    if (n_chunks > max_chunks) return OPTIMI_ERR_SIZE;
+  }
+  if (n_chunks_out) *n_chunks_out = n_chunks;
+  return OPTIMI_OK;
+}
+
+// chunk -> tensor for every chunk of the launch; `map` has room for the launch's chunk count.
+inline void build_chunk_map(const TensorEntry* entries, int n_tensors, int64_t chunk, int32_t* map) {
+  for (int t = 0; t < n_tensors; ++t) {
+    const int64_t c0 = entries[t].first_chunk, c1 = c0 + chunks_of(entries[t].numel, chunk);
+    for (int64_t c = c0; c < c1; ++c) map[c] = t;
+  }
+}
+
+// The tensor that owns chunk `chunk_id` of a short list: the last one whose first chunk is not
+// beyond it.  (A tensor without elements owns no chunk: it shares its first_chunk with its
+// successor, which is later in the table and wins; trailing ones start past the last chunk.)
+OPTIMI_HD int few_lookup(const FewTable& few, int64_t chunk_id) {
+  int tensor = 0;
+  for (int t = 1; t < kFew; ++t)
+    if (t < few.n && few.e[t].first_chunk <= chunk_id) tensor = t;
+  return tensor;
+}
+
+// First element, within its tensor, of the tile that workgroup `sub` of chunk `chunk_id` covers.
+// The tile is [base, base + tile) cut off at the tensor's numel; base >= numel means no work.
+OPTIMI_HD int64_t tile_base(int64_t chunk_id, int sub, int64_t first_chunk, int64_t chunk, int64_t tile) {
+  return (chunk_id - first_chunk) * chunk + (int64_t)sub * tile;
+}
+
+}  // namespace optimi_tables
+
+#endif  // OPTIMI_TABLES_H

@@ -523,8 +523,8 @@ void check_hip(hipError_t err, const char* what) {
 // scalar - which includes the step count through the debiased betas).  A tensor of a few
 // thousand elements costs far more to launch than to update, so a model with thousands of
 // them is bound by launches; one list launch replaces up to `max_tensors` of them.  The queue
-// keeps each parked gradient alive until its launch; `max_total` bounds how many elements
-// that may be.  Results are those of the per-tensor launches, bit for bit.
+// keeps each parked gradient alive until its launch; `max_total` bounds how many bytes of
+// gradients that may be.  Results are those of the per-tensor launches, bit for bit.
 //
 // Steps are parked only while a backward pass runs: the first one parked in a pass registers
 // a final callback with the autograd engine, which launches whatever is parked when the pass
@@ -577,7 +577,7 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
     const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(c.param().device().index()).stream();
     if (!batch_.empty() && (!same_run(c, stream) || seen_.count(c.param().data_ptr()))) flush();
     if (batch_.empty()) stream_ = stream;
-    total_ += c.param().numel();
+    total_ += c.param().numel() * (int64_t)c.param().element_size();
     seen_.insert(c.param().data_ptr());
     batch_.push_back(std::move(c));
     if ((int64_t)batch_.size() >= max_tensors_ || total_ >= max_total_) flush();
@@ -627,7 +627,9 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
       // soon as this function returns: tell the caching allocator that another stream reads them.
       for (const StepCall& c : batch) c.t[1]->record_stream(current_stream);
     }
-    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtype, c0.s, c0.flags, launch);
+    // OPTIMI_COLD: these tensors are a slice of a model whose backward pass has just streamed
+    // through the caches; a short list must not be taken for a small resident model
+    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtype, c0.s, c0.flags | OPTIMI_COLD, launch);
     ++launches_;
     launched_steps_ += n;
     if (launch != current) {
@@ -1185,7 +1187,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.attr("KIND_RADAM") = (int)RADAM;
   mod.attr("KIND_RANGER") = (int)RANGER;
   py::class_<ReleaseQueue, std::shared_ptr<ReleaseQueue>>(mod, "ReleaseQueue")
-      .def(py::init<int64_t, int64_t, int64_t>(), py::arg("max_numel"), py::arg("max_tensors"), py::arg("max_total"))
+      .def(py::init<int64_t, int64_t, int64_t>(), py::arg("max_numel"), py::arg("max_tensors"), py::arg("max_total_bytes"))
       .def("flush", [](ReleaseQueue& q) { q.flush(); })
       .def("pending", &ReleaseQueue::pending)
       .def("launches", &ReleaseQueue::launches)

@@ -54,13 +54,16 @@ class OptimiOptimizer(Optimizer):
     _release_kind = ""                      # name of the native hook's optimizer kind (KIND_* of the extension)
 
     # Gradient release parks the steps of tensors with at most this many elements and launches
-    # them together when the backward pass ends (0 = launch every tensor on its own, from its
-    # hook).  Results are identical; a model with thousands of small tensors steps several times
-    # faster.  Set on the instance, or on the class, before prepare_for_gradient_release.
+    # them together - when the parked gradients reach _QUEUE_MAX_BYTES or _QUEUE_MAX_TENSORS, and
+    # when the backward pass ends (0 = launch every tensor on its own, from its hook).  Results
+    # are identical; a model with thousands of small tensors steps several times faster, and the
+    # attention matrices of a 7B model, launched four at a time, fill the GPU better than one by
+    # one.  The price is that up to _QUEUE_MAX_BYTES of gradients (plus one tensor) stay alive a
+    # little longer.  Set on the instance, or on the class, before prepare_for_gradient_release.
     native_step = True                      # False: walk the parameters in Python on every step (same results)
-    gradient_release_coalesce = 65536
+    gradient_release_coalesce = 1 << 25
     _QUEUE_MAX_TENSORS = 1024               # parked steps per launch
-    _QUEUE_MAX_ELEMENTS = 1 << 24           # parked gradient elements kept alive at most
+    _QUEUE_MAX_BYTES = 128 << 20            # bytes of parked gradients kept alive at most
 
     def __init__(self, params: Iterable[Tensor] | Iterable[dict], defaults: dict[str, Any]):
         if not 0.0 <= defaults["lr"]:
@@ -291,7 +294,7 @@ class OptimiOptimizer(Optimizer):
         """The queue that parks the steps of small tensors during a backward pass, or None."""
         if self._release_queue is None and self.gradient_release_coalesce > 0:
             self._release_queue = backend.ext().ReleaseQueue(self.gradient_release_coalesce, self._QUEUE_MAX_TENSORS,
-                                                             self._QUEUE_MAX_ELEMENTS)
+                                                             self._QUEUE_MAX_BYTES)
         return self._release_queue
 
     def _release_entry(self, param: Tensor):

@@ -255,6 +255,7 @@ def test_coalesced_release_equals_per_tensor_launches(case, max_tensors, hip_dev
     a, b = ManySmall(hip_device), ManySmall(hip_device)
     parked, direct = cls(a.parameters(), gradient_release=True, **hyper), cls(b.parameters(), gradient_release=True, **hyper)
     parked._QUEUE_MAX_TENSORS = max_tensors
+    parked.gradient_release_coalesce = 65536  # ManySmall has tensors on both sides of this limit
     direct.gradient_release_coalesce = 0
     optimi_amd.prepare_for_gradient_release(a, parked)
     optimi_amd.prepare_for_gradient_release(b, direct)

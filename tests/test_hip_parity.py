@@ -232,6 +232,31 @@ def test_empty_and_changing_lists(hip_device):
         G.assert_bits_equal(hip.state[i]["kahan_comp"], sca.state[i]["kahan_comp"], f"kahan {i}")
 
 
+@pytest.mark.parametrize("cfg", ["adamw", "stableadamw", "adan"])
+@pytest.mark.parametrize("n_tensors", [1, 2, 15, 16, 17, 40])
+def test_list_lengths_around_the_kernel_argument_table(cfg, n_tensors, hip_device):
+    """Lists of up to 16 tensors travel as a kernel argument and are searched by the workgroups;
+    longer ones go through the chunk map in device memory.  Both must give the emulator's bits
+    on either side of the switch, with empty tensors in the middle and at the end of the list
+    (they own no chunk) and tensors of one tile, one chunk and several chunks."""
+    hyper, name = CONFIGS[cfg], OPT_OF[cfg]
+    pattern = [8193, 0, 700, 512, 0, 8192, 1, 20000, 3, 0]
+    sizes = [pattern[i % len(pattern)] for i in range(n_tensors)]
+    if n_tensors > 2:
+        sizes[-1] = 0
+    params, grads = draw(sizes, torch.bfloat16, 5, seed=21 + n_tensors)
+    guard = Guarded(hip_device)
+    hip = hip_engine(name, params, hip_device, guard, **hyper)
+    sca = ScalarRun(name, [p.clone() for p in params], **hyper)
+    for t, gs in enumerate(grads):
+        skip = {0} if (t == 2 and n_tensors > 1) else set()  # the list changes length and shifts by one
+        hip.step([None if i in skip else guard(g) for i, g in enumerate(gs)])
+        sca.step([None if i in skip else g.clone() for i, g in enumerate(gs)])
+    torch.cuda.synchronize()
+    guard.check()
+    G.compare_engines(hip, sca, f"{cfg} list of {n_tensors}", exact=name != "stableadamw")
+
+
 def test_rejected_arguments_on_device(hip_device):
     from optimi_amd import cabi
 

@@ -65,11 +65,11 @@ def check_against(opt, params, sca, idxs, what):
         assert p.grad is None
 
 
-@pytest.mark.parametrize("max_elements", [None, 1 << 22], ids=["default_limits", "element_limit_4M"])
-def test_hooks_on_the_10000_tensor_stress_list(max_elements, hip_device):
-    """With the default limits the queue launches every 1024 parked tensors (a pass parks about
-    six times ``_QUEUE_MAX_ELEMENTS`` elements in all, but 1024 average tensors stay below it);
-    with the element limit lowered to 4 M that limit cuts every launch short instead."""
+@pytest.mark.parametrize("max_bytes", [None, 8 << 20], ids=["default_limits", "byte_limit_8M"])
+def test_hooks_on_the_10000_tensor_stress_list(max_bytes, hip_device):
+    """With the default limits the queue launches every 1024 parked tensors (a pass parks more
+    than ``_QUEUE_MAX_BYTES`` of gradients in all, but 1024 average tensors stay below it); with
+    the byte limit lowered to 8 MiB that limit cuts every launch short instead."""
     rng = torch.Generator().manual_seed(6)
     sizes = torch.exp(torch.empty(10_000).uniform_(math.log(128), math.log(65536), generator=rng)).long().clamp(128, 65536).tolist()
     shapes = [(n,) for n in sizes]
@@ -78,10 +78,10 @@ def test_hooks_on_the_10000_tensor_stress_list(max_elements, hip_device):
     model = torch.nn.Module()
     model.ps = torch.nn.ParameterList(params)
     opt = optimi_amd.AdamW(params, gradient_release=True, **ADAMW)
-    if max_elements is not None:
-        opt._QUEUE_MAX_ELEMENTS = max_elements
+    if max_bytes is not None:
+        opt._QUEUE_MAX_BYTES = max_bytes
     optimi_amd.prepare_for_gradient_release(model, opt)
-    assert sum(sizes) > 4 * opt._QUEUE_MAX_ELEMENTS and max(sizes) <= opt.gradient_release_coalesce
+    assert 2 * sum(sizes) > opt._QUEUE_MAX_BYTES and max(sizes) <= opt.gradient_release_coalesce
     by_tensor_limit = math.ceil(len(params) / opt._QUEUE_MAX_TENSORS)
 
     sca = ScalarRun("adamw", [p.detach().cpu() for p in params], gradient_release=True, **ADAMW)
@@ -100,8 +100,8 @@ def test_hooks_on_the_10000_tensor_stress_list(max_elements, hip_device):
         assert queue.launched_steps() - steps_before == len(params)
         flushes = queue.launches() - before
         assert flushes >= by_tensor_limit == 10, flushes
-        if max_elements is not None:  # about 105 M elements per pass, at most 4 M + one tensor per launch
-            assert flushes >= sum(sizes) // (max_elements + 65536) > 2 * by_tensor_limit, flushes
+        if max_bytes is not None:  # about 210 MB of gradients per pass, at most 8 MiB + one tensor per launch
+            assert flushes >= 2 * sum(sizes) // (max_bytes + 2 * 65536) > 2 * by_tensor_limit, flushes
         for i in reversed(range(len(params))):  # the order autograd releases them in does not matter: steps are per tensor
             sca.step_param(i, current[0][i].cpu())
     torch.cuda.synchronize()
@@ -136,7 +136,7 @@ def test_hooks_on_the_llama7b_list(hip_device):
     feed = make_feed(current)
     queue = opt._queue()
     n_small = sum(1 for s in shapes if math.prod(s) <= opt.gradient_release_coalesce)
-    assert n_small == 64  # the norm weights are parked, the matrices launch from their hooks
+    assert n_small == 64 + 128  # norm weights and attention matrices are parked, the rest launch from their hooks
     for t in range(PASSES):
         accumulate = (t + 1) % 4 != 0
         opt.optimizer_accumulation = sca.optimizer_accumulation = accumulate
