@@ -20,11 +20,17 @@ cores on a bounded sample of the same list.
 Two more workloads time gradient release instead (see release_bench):
 ``adamw_bf16_kahan_release_stress10k`` (10,000 small tensors, launch-bound) and
 ``adamw_bf16_kahan_release_llama7b``; ``--no-coalesce`` turns the parking of small tensors off.
+
+Besides the headline workload the line carries ``extra``: the other benchmark configurations
+(the fp32 MLP list, the Llama-1B list, Lion / StableAdamW / Adan on the Llama-7B list, and the two
+gradient-release workloads), each measured the same way in the same process, as
+``{workload: {ms_per_step, kernel_ms, achieved GB/s, frac}}``.  ``--no-extra`` leaves them out.
 """
 
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -68,17 +74,24 @@ def workloads():
     }
 
 
-# HBM bytes per step read off the hardware counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
-# scaled by what the same counters read for a plain copy of known size).  None = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/adamw_bf16_kahan_llama7b_hbm_traffic.txt: 67.44 GB read + 53.90 GB written
-    "adamw_bf16_kahan_llama7b": 1.2134e11,
-    # profiles/lion_stableadamw_adan_adamw1b_hbm_traffic.txt
-    "lion_bf16_kahan_llama7b": 9.439e10,
-    "stableadamw_bf16_kahan_llama7b": 1.4887e11,
-    "adan_bf16_kahan_llama7b": 1.7524e11,
-    "adamw_bf16_kahan_declr_llama1b": 2.170e10,
+# HBM bytes per step read off the hardware counters in a separate profiler run (rocprofv3 --pmc
+# FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the library's plain
+# copy kernel over a known size).  bench.py cannot read the counters itself, so the line quotes
+# the kept profile: workload -> (bytes per step, the file under profiles/ that shows them).
+MEASURED_TRAFFIC = {
+    "adamw_bf16_kahan_llama7b": (1.2134e11, "profiles/adamw_bf16_kahan_llama7b_hbm_traffic.txt"),
+    "lion_bf16_kahan_llama7b": (9.439e10, "profiles/lion_stableadamw_adan_adamw1b_hbm_traffic.txt"),
+    "stableadamw_bf16_kahan_llama7b": (1.4887e11, "profiles/lion_stableadamw_adan_adamw1b_hbm_traffic.txt"),
+    "adan_bf16_kahan_llama7b": (1.7524e11, "profiles/lion_stableadamw_adan_adamw1b_hbm_traffic.txt"),
+    "adamw_bf16_kahan_declr_llama1b": (2.170e10, "profiles/lion_stableadamw_adan_adamw1b_hbm_traffic.txt"),
 }
+
+# the benchmark configurations reported under "extra" next to the headline workload
+EXTRA_WORKLOADS = [
+    "adamw_fp32_mlp", "adamw_bf16_kahan_declr_llama1b", "lion_bf16_kahan_llama7b", "stableadamw_bf16_kahan_llama7b",
+    "adan_bf16_kahan_llama7b", "adamw_bf16_kahan_release_llama7b", "adamw_bf16_kahan_release_stress10k",
+]
+RELEASE_WORKLOADS = ("adamw_bf16_kahan_release_stress10k", "adamw_bf16_kahan_release_llama7b")
 
 
 def numel(shape):
@@ -103,38 +116,47 @@ def make_tensors(shapes, dtype, device, seed, std, ones_for_1d=False):
     return out
 
 
-def cpu_baseline(cls_name, kwargs, dtype, shapes, budget_s=20.0):
-    """Times the for-loop restatement on a bounded sample: the tensors of one transformer layer
-    (or the whole list when it is small)."""
+def cpu_baseline(cls_name, kwargs, dtype, shapes, budget_s=25.0):
+    """Times the for-loop restatement on the host: the whole list when it is small, otherwise every
+    distinct shape of the list on its own (1 warm-up, then the median of up to 5 steps), the
+    list's time being the sum over shapes of time x multiplicity."""
     import torch
 
     from oracle.forloop import ForLoopRun
 
-    total = sum(numel(s) for s in shapes)
-    sample = shapes if total <= 64_000_000 else shapes[1:10]
-    what = "whole list" if sample is shapes else "one transformer layer (tensors 1-9 of the list)"
-    n = sum(numel(s) for s in sample)
     name = cls_name.lower()
-    params = make_tensors(sample, dtype, "cpu", 1, 0.02, ones_for_1d=True)
-    grads = make_tensors(sample, dtype, "cpu", 2, 1e-3)
-    run = ForLoopRun(name, params, **kwargs)
-    run.step([g.clone() for g in grads])  # warm-up, creates the states
-    times = []
+    total = sum(numel(s) for s in shapes)
+    counts = {}
+    for s in shapes:
+        counts[s] = counts.get(s, 0) + 1
+    groups = [(list(shapes), 1)] if total <= 64_000_000 else [([s], c) for s, c in counts.items()]
+    list_seconds, n_steps = 0.0, 0
     t_begin = time.perf_counter()
-    while len(times) < 3 or (len(times) < 10 and time.perf_counter() - t_begin < budget_s / 2):
-        gs = [g.clone() for g in grads]  # the for-loop path uses grad as scratch
-        t0 = time.perf_counter()
-        run.step(gs)
-        times.append(time.perf_counter() - t0)
-        if time.perf_counter() - t_begin > budget_s:
-            break
-    per_step = sorted(times)[len(times) // 2]
+    for sample, mult in groups:
+        params = make_tensors(sample, dtype, "cpu", 1, 0.02, ones_for_1d=True)
+        grads = make_tensors(sample, dtype, "cpu", 2, 1e-3)
+        run = ForLoopRun(name, params, **kwargs)
+        run.step([g.clone() for g in grads])  # warm-up, creates the states
+        times = []
+        while len(times) < 5:
+            gs = [g.clone() for g in grads]  # the for-loop path uses grad as scratch
+            t0 = time.perf_counter()
+            run.step(gs)
+            times.append(time.perf_counter() - t0)
+            if len(times) >= 2 and time.perf_counter() - t_begin > budget_s * (n_steps + len(times)) / (n_steps + len(times) + 3):
+                break
+        list_seconds += mult * sorted(times)[len(times) // 2]
+        n_steps += len(times)
+        del run, params, grads
+    what = ("whole list" if len(groups) == 1 else
+            f"each of the {len(groups)} distinct shapes timed on its own, summed with its multiplicity")
     return {
-        "value": n / per_step,
+        "value": total / list_seconds,
         "unit": "params/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{what}: {n} params, median of {len(times)} steps after 1 warm-up, host has {os.cpu_count()} logical CPUs",
+        "sample": f"{what}: {total} params, {list_seconds * 1e3:.1f} ms per step of the list, median of up to 5 steps per shape after "
+                  f"1 warm-up ({n_steps} timed steps), host has {os.cpu_count()} logical CPUs",
     }
 
 
@@ -149,7 +171,7 @@ def stress_shapes(n_tensors=10_000, lo=128, hi=65536, seed=6):
     return [(int(n),) for n in torch.exp(u).long().clamp(lo, hi).tolist()]
 
 
-def release_bench(args):
+def release_bench(workload, args, steps, warmup):
     """Gradient release: AdamW bf16 + Kahan stepped per tensor from real post-accumulate-grad hooks,
     in cycles of 3 accumulate-only backward passes and 1 full one.  An autograd function hands
     pre-made gradients to the parameters, so the backward pass launches no kernels of its own and
@@ -160,7 +182,7 @@ def release_bench(args):
     import optimi_amd
 
     device = torch.device("cuda:0")
-    shapes = stress_shapes() if args.workload.endswith("stress10k") else llama_shapes(4096, 11008, 32)
+    shapes = stress_shapes() if workload.endswith("stress10k") else llama_shapes(4096, 11008, 32)
     n_params = sum(numel(s) for s in shapes)
     params = [torch.nn.Parameter(p) for p in make_tensors(shapes, torch.bfloat16, device, 0, 0.02, ones_for_1d=True)]
     grads = make_tensors(shapes, torch.bfloat16, device, 100, 1e-3)
@@ -204,29 +226,130 @@ def release_bench(args):
         opt.optimizer_accumulation = (i + 1) % 4 != 0
         Feed.apply(*params).backward()
 
-    for i in range(args.warmup):
+    for i in range(warmup):
         one_pass(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        one_pass(args.warmup + i)
+    for i in range(steps):
+        one_pass(warmup + i)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    full = sum(1 for i in range(args.steps) if (args.warmup + i + 1) % 4 == 0)
-    algo_bytes = n_params * (18.0 * full + 10.0 * (args.steps - full))
+    full = sum(1 for i in range(steps) if (warmup + i + 1) % 4 == 0)
+    algo_bytes = n_params * (18.0 * full + 10.0 * (steps - full))
     achieved = algo_bytes / elapsed / 1e9
-    print(json.dumps({
+    optimi_amd.remove_gradient_release(model)
+    out = {
         "metric": "gradient-release tensor-steps/s (AdamW bf16 Kahan, accumulation_steps=4)",
-        "value": len(shapes) * args.steps / elapsed, "unit": "tensor-steps/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "value": len(shapes) * steps / elapsed, "unit": "tensor-steps/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": elapsed / steps * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": args.workload, "optimizer": "AdamW", "n_tensors": len(shapes), "n_params": n_params,
+        "config": {"workload": workload, "optimizer": "AdamW", "n_tensors": len(shapes), "n_params": n_params,
                    "coalesce": opt.gradient_release_coalesce, "empty_hook_pass_ms": floor_ms,
-                   "us_per_tensor_over_empty_hook": (elapsed / args.steps * 1e3 - floor_ms) * 1e3 / len(shapes), "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()}},
+                   "us_per_tensor_over_empty_hook": (elapsed / steps * 1e3 - floor_ms) * 1e3 / len(shapes), "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": None, "note": "wall-clock over whole backward passes, launch-bound for small tensors"},
+                     "traffic": None, "traffic_source": None,
+                     "note": "wall clock over whole backward passes (hook dispatch included), launch-bound for small tensors; "
+                             "a step is one backward pass, 3 of 4 accumulate-only (10 B/param), 1 of 4 full (18 B/param)"},
         "cpu_baseline": None,
-    }), flush=True)
+    }
+    del opt, params, grads, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def list_bench(workload, args, steps, warmup):
+    """One whole-list optimizer step per "step", through the optimizer class."""
+    import torch
+
+    import optimi_amd
+
+    device = torch.device("cuda:0")
+    cls_name, kwargs, dtype_name, shapes, bytes_per_param = workloads()[workload]
+    dtype = getattr(torch, dtype_name)
+    n_params = sum(numel(s) for s in shapes)
+
+    params = [torch.nn.Parameter(p) for p in make_tensors(shapes, dtype, device, 0, 0.02, ones_for_1d=True)]
+    grad_sets = [make_tensors(shapes, dtype, device, 100 + i, 1e-3) for i in range(max(1, args.grad_sets))]
+    opt = getattr(optimi_amd, cls_name)(params, **kwargs)
+
+    def one_step(i):
+        for p, g in zip(params, grad_sets[i % len(grad_sets)]):
+            p.grad = g
+        opt.step()
+
+    for i in range(warmup):
+        one_step(i)
+    torch.cuda.synchronize()
+
+    # HIP events on the stream the kernels are launched on (torch's current stream is the one the
+    # binding hands to the library)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        one_step(warmup + i)
+        stops[i].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kernel_ms = [a.elapsed_time(b) for a, b in zip(starts, stops)]
+    mean_kernel_ms = sum(kernel_ms) / len(kernel_ms)
+
+    if cls_name == "Ranger":  # average over the timed steps, of which every k-th is a Lookahead step
+        k = kwargs["k"]
+        slow = sum(1 for t in range(warmup + 1, warmup + steps + 1) if t % k == 0)
+        bytes_per_param += 4.0 * slow / steps
+    algo_bytes = bytes_per_param * n_params
+    achieved = algo_bytes / (mean_kernel_ms * 1e-3) / 1e9
+    traffic, source = MEASURED_TRAFFIC.get(workload, (None, None))
+    out = {
+        "metric": "optimizer-step params/sec + achieved HBM GB/s (% of peak), bf16 Kahan AdamW 6.7B",
+        "value": n_params * steps / elapsed,
+        "unit": "params/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": elapsed / steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype],
+        "data": "synthetic",
+        "config": {"workload": workload, "optimizer": cls_name, "n_tensors": len(shapes), "n_params": n_params,
+                   "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()},
+                   "grad_sets": len(grad_sets)},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": source,
+                     "bytes_per_param": bytes_per_param, "kernel_ms": mean_kernel_ms,
+                     "kernel_ms_min": min(kernel_ms), "kernel_ms_max": max(kernel_ms),
+                     "kernel_ms_p50": sorted(kernel_ms)[len(kernel_ms) // 2],
+                     "kernel_ms_p90": sorted(kernel_ms)[min(len(kernel_ms) - 1, (len(kernel_ms) * 9) // 10)]},
+        "cpu_baseline": None,
+    }
+    if traffic is None:
+        out["roofline"]["traffic_note"] = "no hardware-counter profile is kept for this workload"
+    del opt, params, grad_sets
+    torch.cuda.empty_cache()
+    return out, (cls_name, kwargs, dtype, shapes)
+
+
+def run_workload(workload, args, steps, warmup):
+    if workload in RELEASE_WORKLOADS:
+        return release_bench(workload, args, steps, warmup), None
+    return list_bench(workload, args, steps, warmup)
+
+
+def brief(line):
+    """The part of a workload's line that goes under "extra"."""
+    r = line["roofline"]
+    out = {"ms_per_step": line["ms_per_step"], "achieved_gbps": r["achieved"], "frac": r["frac"], "steps": line["steps"],
+           "unit": line["unit"], "value": line["value"]}
+    if "kernel_ms" in r:
+        out.update(kernel_ms=r["kernel_ms"], kernel_ms_min=r["kernel_ms_min"], bytes_per_param=r["bytes_per_param"])
+    else:
+        out.update(timed="wall clock over backward passes", empty_hook_pass_ms=line["config"]["empty_hook_pass_ms"])
+    return out
 
 
 def main():
@@ -237,6 +360,7 @@ def main():
     ap.add_argument("--workload", default="adamw_bf16_kahan_llama7b")
     ap.add_argument("--grad-sets", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="measure the named workload only, not the other configurations")
     ap.add_argument("--no-coalesce", action="store_true",
                     help="gradient-release workloads: launch every tensor from its own hook instead of parking small ones")
     ap.add_argument("--copy-probe-bytes", type=int, default=0,
@@ -254,7 +378,7 @@ def main():
 
     import torch
 
-    import optimi_amd
+    import optimi_amd  # noqa: F401  (fails loudly here when the HIP extension is missing)
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no HIP device visible")
@@ -270,73 +394,24 @@ def main():
                        "optimi_hip_copy_probe")
         torch.cuda.synchronize()
         del src, dst
-    if args.workload in ("adamw_bf16_kahan_release_stress10k", "adamw_bf16_kahan_release_llama7b"):
-        return release_bench(args)
-    cls_name, kwargs, dtype_name, shapes, bytes_per_param = workloads()[args.workload]
-    dtype = getattr(torch, dtype_name)
-    n_params = sum(numel(s) for s in shapes)
 
-    params = [torch.nn.Parameter(p) for p in make_tensors(shapes, dtype, device, 0, 0.02, ones_for_1d=True)]
-    grad_sets = [make_tensors(shapes, dtype, device, 100 + i, 1e-3) for i in range(max(1, args.grad_sets))]
-    opt = getattr(optimi_amd, cls_name)(params, **kwargs)
-
-    def one_step(i):
-        for p, g in zip(params, grad_sets[i % len(grad_sets)]):
-            p.grad = g
-        opt.step()
-
-    for i in range(args.warmup):
-        one_step(i)
-    torch.cuda.synchronize()
-
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        starts[i].record()
-        one_step(args.warmup + i)
-        stops[i].record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    kernel_ms = [a.elapsed_time(b) for a, b in zip(starts, stops)]
-    mean_kernel_ms = sum(kernel_ms) / len(kernel_ms)
-
-    if cls_name == "Ranger":  # average over the timed steps, of which every k-th is a Lookahead step
-        k = kwargs["k"]
-        slow = sum(1 for t in range(args.warmup + 1, args.warmup + args.steps + 1) if t % k == 0)
-        bytes_per_param += 4.0 * slow / args.steps
-    algo_bytes = bytes_per_param * n_params
-    achieved = algo_bytes / (mean_kernel_ms * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
-    out = {
-        "metric": "optimizer-step params/sec + achieved HBM GB/s (% of peak), bf16 Kahan AdamW 6.7B",
-        "value": n_params * args.steps / elapsed,
-        "unit": "params/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": elapsed / args.steps * 1e3,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype],
-        "data": "synthetic",
-        "config": {"workload": args.workload, "optimizer": cls_name, "n_tensors": len(shapes), "n_params": n_params,
-                   "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()},
-                   "grad_sets": len(grad_sets)},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
-                     "bytes_per_param": bytes_per_param, "kernel_ms": mean_kernel_ms,
-                     "kernel_ms_min": min(kernel_ms), "kernel_ms_max": max(kernel_ms),
-                     "kernel_ms_p50": sorted(kernel_ms)[len(kernel_ms) // 2],
-                     "kernel_ms_p90": sorted(kernel_ms)[min(len(kernel_ms) - 1, (len(kernel_ms) * 9) // 10)]},
-        "cpu_baseline": None,
-    }
-    del opt, params, grad_sets
+    out, spec = run_workload(args.workload, args, args.steps, args.warmup)
+    gc.collect()
     torch.cuda.empty_cache()
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cls_name, kwargs, dtype, shapes)
+    if not args.no_extra:
+        extra = {}
+        for name in EXTRA_WORKLOADS:
+            if name == args.workload:
+                continue
+            # short launches are timed over more steps: a 0.1 ms step needs many to average the host's jitter out
+            steps = 200 if name == "adamw_fp32_mlp" else (40 if "llama1b" in name else (16 if name in RELEASE_WORKLOADS else 12))
+            line, _ = run_workload(name, args, steps, 8 if name in RELEASE_WORKLOADS else 5)
+            extra[name] = brief(line)
+            gc.collect()
+            torch.cuda.empty_cache()
+        out["extra"] = extra
+    if spec is not None and not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(*spec)
     print(json.dumps(out), flush=True)
 
 

@@ -65,12 +65,18 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 // Pointers come out of the tensor table as plain addresses; telling the compiler they are
 // global memory gets global_load/global_store instead of flat accesses.
 #define OPTIMI_GLOBAL __attribute__((address_space(1)))
-// `streaming`: the data will not be used again before it has left every cache (`nt` policy).
-// Without it the load is an ordinary cached one, which is what a working set small enough to
-// stay in the 256 MB last-level cache between steps wants.  The flag is wave-uniform.
-__device__ __forceinline__ u32x4 load16(const void* base, int64_t byte_off, bool streaming) {
-  const OPTIMI_GLOBAL u32x4* p = (const OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off);
-  return streaming ? __builtin_nontemporal_load(p) : *p;
+// Streaming load: the data will not be used again before it has left every cache (`nt` policy).
+__device__ __forceinline__ u32x4 load16(const void* base, int64_t byte_off) {
+  return __builtin_nontemporal_load((const OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
+}
+// Ordinary cached load of a lane's vector of a full tile, for a working set small enough to stay
+// in the 256 MB last-level cache between steps.  Written as a buffer load so that the compiler
+// cannot merge it with the streaming load of the other branch (merging two loads that differ only
+// in the `nt` hint drops the hint from both).  `tile` (wave-uniform) points at the workgroup's
+// tile of one array, `lane_off` is the lane's byte offset in it.
+__device__ __forceinline__ u32x4 load16_tile_cached(const void* tile, uint32_t lane_off) {
+  __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(tile), 0, (uint32_t)(kThreads * kUnroll * 16), 0x00020000);
+  return __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, 0, 0);
 }
 __device__ __forceinline__ void store16(void* base, int64_t byte_off, u32x4 v) {
   __builtin_nontemporal_store(v, (OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
@@ -564,17 +570,22 @@ __device__ __forceinline__ void compute_store(const TensorEntry& e, int64_t off,
 }
 
 template <class Op>
-__device__ __forceinline__ void load_vec(const TensorEntry& e, int64_t off, u32x4* raw, bool streaming) {
+__device__ __forceinline__ void load_vec(const TensorEntry& e, int64_t off, u32x4* raw) {
   using DT = typename Op::DT;
-  if (streaming) {
 #pragma unroll
-    for (int a = 0; a < Op::kArrays; ++a)
-      if (Op::kLoad & bit(a)) raw[a] = load16(e.ptr[a], off * DT::kElemBytes, true);
-  } else {
+  for (int a = 0; a < Op::kArrays; ++a)
+    if (Op::kLoad & bit(a)) raw[a] = load16(e.ptr[a], off * DT::kElemBytes);
+}
+
+// The same for a lane of a full tile that starts at element `tile_base`, with cached loads.
+template <class Op>
+__device__ __forceinline__ void load_vec_cached(const TensorEntry& e, int64_t off, int64_t tile_base, u32x4* raw) {
+  using DT = typename Op::DT;
 #pragma unroll
-    for (int a = 0; a < Op::kArrays; ++a)
-      if (Op::kLoad & bit(a)) raw[a] = load16(e.ptr[a], off * DT::kElemBytes, false);
-  }
+  for (int a = 0; a < Op::kArrays; ++a)
+    if (Op::kLoad & bit(a))
+      raw[a] = load16_tile_cached((const void*)((uintptr_t)e.ptr[a] + (uintptr_t)(tile_base * DT::kElemBytes)),
+                                  (uint32_t)((off - tile_base) * DT::kElemBytes));
 }
 
 template <class Op>
@@ -592,16 +603,13 @@ __device__ __forceinline__ void one_element(const TensorEntry& e, int64_t i, con
     if (Op::kStore & bit(a)) DT::store1(e.ptr[a], i, x[a].x);
 }
 
-// Launch policy bits (kernel argument).
-constexpr uint32_t kPolicyCachedLoads = 1;  // ordinary cached loads instead of `nt` ones
-
 // MULTI: the tensor table and the chunk map are in device memory.  Otherwise the table travels
 // as the kernel argument `few` (one tensor for the per-tensor entry points, up to kFew for
 // short lists) and the workgroup searches it.
 template <class Op, bool MULTI>
 __global__ void __launch_bounds__(kThreads)
 step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, const FewTable few,
-            typename Op::Scalars s, double* __restrict__ partials, uint32_t policy) {
+            typename Op::Scalars s, double* __restrict__ partials) {
   using DT = typename Op::DT;
   constexpr int V = DT::kVec;
   constexpr int A = Op::kArrays;
@@ -610,30 +618,41 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
 
   const int64_t chunk_id = blockIdx.x / kSub;
   const int sub = blockIdx.x % kSub;
-  const int tensor = MULTI ? chunk_map[chunk_id] : optimi_tables::few_lookup(few, chunk_id);
+  // a table of one (the per-tensor entry points) needs no search
+  const int tensor = MULTI ? chunk_map[chunk_id] : (few.n == 1 ? 0 : optimi_tables::few_lookup(few, chunk_id));
   const TensorEntry& e = MULTI ? table[tensor] : few.e[tensor];
   const int64_t base = optimi_tables::tile_base(chunk_id, sub, e.first_chunk, kChunk, kTile);
   const int64_t remain = e.numel - base;  // <= 0 for tiles past the end of the tensor's last chunk
-  const bool streaming = !(policy & kPolicyCachedLoads);
+  const bool vec_ok = (e.flags & optimi_tables::kEntryVec) != 0;
   Op::prepare(s, tensor);
 
   float acc = 0.0f;
-  if (e.vec_ok && remain >= kTile) {
-    // full tile: every load is issued before the first use
-    u32x4 raw[kUnroll][A];
+  if (vec_ok && remain >= kTile) {
+    // full tile: every load is issued before the first use.  The two cache policies are two
+    // copies of the whole tile body, so that each keeps its own schedule of waits.
+    if (e.flags & optimi_tables::kEntryCached) {
+      u32x4 raw[kUnroll][A];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) load_vec<Op>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u], streaming);
+      for (int u = 0; u < kUnroll; ++u) load_vec_cached<Op>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, base, raw[u]);
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      compute_store<Op, true>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u], s, acc, base);
-  } else if (e.vec_ok) {
+      for (int u = 0; u < kUnroll; ++u)
+        compute_store<Op, true>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u], s, acc, base);
+    } else {
+      u32x4 raw[kUnroll][A];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) load_vec<Op>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u]);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        compute_store<Op, true>(e, base + ((int64_t)u * kThreads + threadIdx.x) * V, raw[u], s, acc, base);
+    }
+  } else if (vec_ok) {
     // end of a tensor: whole vectors while they fit, then the few leftover elements
     const int64_t end = e.numel;
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t off = base + ((int64_t)u * kThreads + threadIdx.x) * V;
       if (off + V <= end) {
         u32x4 raw[A];
-        load_vec<Op>(e, off, raw, streaming);
+        load_vec<Op>(e, off, raw);
         compute_store<Op>(e, off, raw, s, acc);
       } else {
         for (int64_t i = off; i < end; ++i) one_element<Op>(e, i, s, acc);
@@ -808,14 +827,24 @@ int staged_upload(optimi_group* g, void* dst, const void* src, size_t bytes, hip
 
 int check_ptrs(int n_tensors, const void* const* list) { return (n_tensors > 0 && list == nullptr) ? OPTIMI_ERR_NULL : 0; }
 
+// A list whose arrays add up to at most this many bytes stays in the 256 MB last-level cache
+// from one optimizer step to the next (measured: cached loads beat `nt` loads up to 270 MB of
+// arrays and lose from 335 MB on).  Such a launch - unless the caller marks it OPTIMI_COLD -
+// uses cached loads and, being short, 21 resident workgroups per CU (16.8 M fp32 parameters in
+// one launch: 83 us -> 78 us).  Per-tensor entry points never take this path: they step one
+// tensor of a larger model, which was last touched a whole backward pass ago (measured on
+// tensors that are cold when revisited: `nt` loads and the table's occupancy are 6-8 % faster
+// there than cached loads or 21 workgroups).
+constexpr int64_t kResidentBytes = (int64_t)288 << 20;
+constexpr int kResidentGranules = 6;
+
 // What one list launch works on, as the entry points hand it to the launchers.
 struct ListPlan {
   bool few = false;           // the table travels as a kernel argument; the group's tables are untouched
   FewTable table;             // valid when `few`
   int n_tensors = 0;
   int64_t n_chunks = 0;
-  int64_t footprint = 0;      // bytes of all arrays the launch touches
-  bool cold = false;          // the caller said the tensors were not touched recently (OPTIMI_COLD)
+  bool resident = false;      // the list's arrays fit the last-level cache and were touched recently
 };
 
 constexpr int64_t kMaxChunks = (int64_t)0x7fffffff / kSub;  // the grid is chunks x kSub workgroups
@@ -835,7 +864,6 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
 
   const int64_t chunk = chunk_elems_rt(dtype);
   plan->n_tensors = n_tensors;
-  plan->cold = (flags & OPTIMI_COLD) != 0;
   plan->few = n_tensors <= kFew;
   std::memset(&plan->table, 0, sizeof(plan->table));
   std::vector<TensorEntry> fresh;
@@ -854,9 +882,11 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
   plan->n_chunks = n_chunks;
   int64_t total = 0;
   for (int t = 0; t < n_tensors; ++t) total += numel[t];
-  plan->footprint = total * elem_bytes(dtype) * popcount(need);
+  plan->resident = !(flags & OPTIMI_COLD) && total * elem_bytes(dtype) * popcount(need) <= kResidentBytes;
+  if (plan->resident)
+    for (int t = 0; t < n_tensors; ++t) entries[t].flags |= optimi_tables::kEntryCached;
   if (plan->few) {
-    plan->table.n = n_tensors;
+    optimi_tables::finish_few(&plan->table, n_tensors);
     return 0;
   }
 
@@ -927,25 +957,14 @@ int finish_list(optimi_group* g, const ListPlan& plan, hipStream_t stream) {
 // The table holds the measured optimum in granules on MI355X with the write-through tile stores
 // (7B-parameter lists; 5 streams = StableAdamW pass 1 and accumulate-only Adam, 6 = pass 2,
 // 7 = Lion / SGD, 9 = Adam with Kahan, 13 = Adan; entries in between are interpolated).  fp32
-// lists with 7 streams do best at 12 workgroups instead of 11.  16-bit launches of fewer than
-// kLongLaunch workgroups (the Llama-1B-shaped list, single tensors) do best one granule lower,
-// i.e. with one more workgroup resident.  OPTIMI_HIP_WAVES overrides the number of wavefronts
+// lists with 7 streams do best at 12 workgroups instead of 11.  16-bit list launches of fewer
+// than kLongLaunch workgroups (the Llama-1B-shaped list) do best one granule lower, i.e. with
+// one more workgroup resident.  OPTIMI_HIP_WAVES overrides the number of wavefronts
 // per CU for every kernel (nearest reachable count at or above it; 0 = no throttle); read once.
 constexpr int kLdsGranule = 1280, kLdsGranules = 128;
 constexpr int kMaxStreams = 2 * kMaxArrays;
 constexpr int kBestGranules[kMaxStreams + 1] = {4, 4, 4, 4, 6, 8, 8, 11, 11, 12, 13, 14, 16, 16, 16};
 constexpr int64_t kLongLaunch = (int64_t)1 << 22;  // workgroups
-
-// A list whose arrays add up to at most this many bytes stays in the 256 MB last-level cache
-// from one optimizer step to the next (measured: cached loads beat `nt` loads up to 270 MB of
-// arrays and lose from 335 MB on).  Such a launch - unless the caller marks it OPTIMI_COLD -
-// uses cached loads and, being short, 21 resident workgroups per CU (16.8 M fp32 parameters in
-// one launch: 83 us -> 78 us).  Per-tensor entry points never take this path: they step one
-// tensor of a larger model, which was last touched a whole backward pass ago (measured on
-// tensors that are cold when revisited: `nt` loads and the table's occupancy are 6-8 % faster
-// there than cached loads or 21 workgroups).
-constexpr int64_t kResidentBytes = (int64_t)288 << 20;
-constexpr int kResidentGranules = 6;
 
 int forced_waves() {
 #ifdef OPTIMI_TUNING
@@ -960,19 +979,24 @@ int forced_waves() {
 }
 
 struct LaunchShape {
-  unsigned lds;     // dynamic LDS request in bytes (the occupancy throttle)
-  uint32_t policy;  // kPolicy* bits
+  unsigned lds;  // dynamic LDS request in bytes (the occupancy throttle)
 };
 
+// `few`: the table travels as a kernel argument (per-tensor launches and short lists).  Such a
+// workgroup reaches its loads sooner than one that first reads the chunk map and the tensor
+// table from memory, so fewer of the resident wavefronts are idle at any time and the optimum
+// sits a little lower: the table as it is for 7 streams and more (no extra workgroup for
+// launches under kLongLaunch), 9 granules instead of 8 for 5 and 6 streams (measured on
+// per-tensor launches over tensors that are cold when revisited, 4 M to 45 M elements).
 template <class Op>
-LaunchShape launch_shape(int64_t workgroups, bool resident) {
+LaunchShape launch_shape(int64_t workgroups, bool resident, bool few) {
   constexpr int streams = (popcount(Op::kLoad) + popcount(Op::kStore)) * kUnroll;
   constexpr bool f32 = std::is_same<typename Op::DT, F32>::value;
   LaunchShape shape;
-  shape.policy = resident ? kPolicyCachedLoads : 0u;
   int granules = kBestGranules[streams < kMaxStreams ? streams : kMaxStreams];
   if (f32 && streams == 7) granules = 10;
-  if (!f32 && streams >= 7 && workgroups < kLongLaunch) granules -= 1;
+  if (!few && !f32 && streams >= 7 && workgroups < kLongLaunch) granules -= 1;
+  if (few && (streams == 5 || streams == 6)) granules = 9;
   if (resident) granules = kResidentGranules;
 #ifdef OPTIMI_TUNING
   if (const char* env = std::getenv("OPTIMI_HIP_LDS")) {  // raw request, tuning builds only
@@ -1003,20 +1027,20 @@ template <class Op>
 void launch_list(optimi_group* g, const ListPlan& plan, const typename Op::Scalars& s, hipStream_t stream,
                  double* partials = nullptr) {
   const int64_t workgroups = plan.n_chunks * kSub;
-  const LaunchShape shape = launch_shape<Op>(workgroups, !plan.cold && plan.footprint <= kResidentBytes);
+  const LaunchShape shape = launch_shape<Op>(workgroups, plan.resident, plan.few);
   if (plan.few)
     step_kernel<Op, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
-        nullptr, nullptr, plan.table, s, partials, shape.policy);
+        nullptr, nullptr, plan.table, s, partials);
   else
     step_kernel<Op, true><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
-        (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, partials, shape.policy);
+        (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, partials);
 }
 
 inline FewTable table_of_one(const TensorEntry& e) {
   FewTable one = {};
   one.e[0] = e;
   one.e[0].first_chunk = 0;
-  one.n = 1;
+  optimi_tables::finish_few(&one, 1);
   return one;
 }
 
@@ -1024,9 +1048,9 @@ template <class Op>
 void launch_single(const TensorEntry& e, const typename Op::Scalars& s, double* partials, hipStream_t stream) {
   const int64_t chunk = chunk_elems<typename Op::DT>();
   const int64_t workgroups = (e.numel + chunk - 1) / chunk * kSub;
-  const LaunchShape shape = launch_shape<Op>(workgroups, false);
+  const LaunchShape shape = launch_shape<Op>(workgroups, false, true);
   step_kernel<Op, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
-      nullptr, nullptr, table_of_one(e), s, partials, shape.policy);
+      nullptr, nullptr, table_of_one(e), s, partials);
 }
 
 // Calls fn(Op{}) for the Op selected by dtype x kahan x update x weight-decay mode.  NWD is
@@ -1087,14 +1111,14 @@ int single_entry(TensorEntry& e, const void* const* ptrs, int n_arrays, uint32_t
   if (numel > chunk_elems_rt(dtype) * ((int64_t)0x7fffffff / kSub)) return OPTIMI_ERR_SIZE;
   std::memset(&e, 0, sizeof(e));
   e.numel = numel;
-  e.vec_ok = 1;
+  e.flags = optimi_tables::kEntryVec;
   const int eb = elem_bytes(dtype);
   for (int a = 0; a < n_arrays; ++a) {
     if (!(need & bit(a))) continue;
     if (!ptrs[a] && numel > 0) return OPTIMI_ERR_NULL;
     uintptr_t u = (uintptr_t)ptrs[a];
     if (u % (uintptr_t)eb) return OPTIMI_ERR_ALIGN;
-    if (u % 16) e.vec_ok = 0;
+    if (u % 16) e.flags &= ~optimi_tables::kEntryVec;
     e.ptr[a] = const_cast<void*>(ptrs[a]);
   }
   return 0;

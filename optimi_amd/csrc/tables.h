@@ -13,6 +13,7 @@
 #ifndef OPTIMI_TABLES_H
 #define OPTIMI_TABLES_H
 
+#include <climits>
 #include <cstdint>
 #include <cstring>
 
@@ -34,13 +35,16 @@ struct TensorEntry {
   void* ptr[kMaxArrays];
   int64_t numel;
   int64_t first_chunk;  // index of this tensor's first chunk within the launch
-  uint32_t vec_ok;      // all buffers 16-byte aligned
+  uint32_t flags;       // kEntry* bits
   uint32_t pad;
 };
+constexpr uint32_t kEntryVec = 1;     // all buffers 16-byte aligned: the vector path applies
+constexpr uint32_t kEntryCached = 2;  // read full tiles with ordinary cached loads instead of streaming ones
 static_assert(sizeof(TensorEntry) == 80, "TensorEntry layout");
 
 struct FewTable {
   TensorEntry e[kFew];
+  int32_t first_chunk[kFew];  // e[t].first_chunk again, packed so that one scalar load fetches all; INT32_MAX from n on
   int32_t n;
   int32_t pad;
 };
@@ -73,14 +77,14 @@ inline int build_entries(int n_tensors, const void* const* const* lists, int n_a
     if (numel[t] > max_chunks * chunk) return OPTIMI_ERR_SIZE;  // also keeps the sums below from overflowing
     e.numel = numel[t];
     e.first_chunk = n_chunks;
-    e.vec_ok = 1;
+    e.flags = kEntryVec;
     for (int a = 0; a < n_arrays; ++a) {
       if (!(need & bit(a))) continue;
       const void* p = lists[a][t];
       if (!p && numel[t] > 0) return OPTIMI_ERR_NULL;
       const uintptr_t u = (uintptr_t)p;
       if (u % eb) return OPTIMI_ERR_ALIGN;
-      if (u % 16) e.vec_ok = 0;
+      if (u % 16) e.flags &= ~kEntryVec;
       e.ptr[a] = const_cast<void*>(p);
     }
     n_chunks += chunks_of(numel[t], chunk);
@@ -98,14 +102,25 @@ inline void build_chunk_map(const TensorEntry* entries, int n_tensors, int64_t c
   }
 }
 
+// Fills the packed search keys of a short list from its entries.
+inline void finish_few(FewTable* few, int n_tensors) {
+  few->n = n_tensors;
+  for (int t = 0; t < kFew; ++t)
+    few->first_chunk[t] = t < n_tensors ? (int32_t)few->e[t].first_chunk : INT32_MAX;
+}
+
 // The tensor that owns chunk `chunk_id` of a short list: the last one whose first chunk is not
-// beyond it.  (A tensor without elements owns no chunk: it shares its first_chunk with its
+// beyond it, i.e. the count of such tensors minus one - sixteen compares on one 64-byte load, no
+// branches.  (A tensor without elements owns no chunk: it shares its first_chunk with its
 // successor, which is later in the table and wins; trailing ones start past the last chunk.)
 OPTIMI_HD int few_lookup(const FewTable& few, int64_t chunk_id) {
-  int tensor = 0;
-  for (int t = 1; t < kFew; ++t)
-    if (t < few.n && few.e[t].first_chunk <= chunk_id) tensor = t;
-  return tensor;
+  // first_chunk[t] <= chunk_id  <=>  first_chunk[t] - chunk_id - 1 < 0; both are below 2^31 / 16,
+  // so the difference cannot wrap and its sign bit is the comparison (plain integer arithmetic
+  // keeps the whole search in scalar registers)
+  const int32_t c = (int32_t)chunk_id;
+  uint32_t count = 0;
+  for (int t = 0; t < kFew; ++t) count += (uint32_t)(few.first_chunk[t] - c - 1) >> 31;
+  return (int)count - 1;
 }
 
 // First element, within its tensor, of the tile that workgroup `sub` of chunk `chunk_id` covers.
