@@ -4,11 +4,12 @@
 // (param, grad, moments, Kahan buffer).  Tensors are cut into chunks of 16 KiB per array;
 // kSub workgroups of kThreads lanes share a chunk, each lane issuing kUnroll 16-byte loads
 // per array before the first use, doing the arithmetic in fp32 registers and writing
-// 16-byte stores back in place.  A whole parameter list runs as ONE launch: a chunk map
-// (chunk -> tensor) and a tensor table (pointers, size, first chunk) tell each workgroup
-// where it works.  How many workgroups a CU holds at once is throttled with a dummy
-// dynamic-LDS request (see throttle_lds): with up to thirteen concurrent streams HBM runs
-// best when only a few tens of KiB per CU are in flight.
+// 16-byte stores back in place.  A whole parameter list runs as ONE launch: a tensor table
+// (pointers, size, first chunk) tells each workgroup where it works - found through a chunk
+// map (chunk -> tensor) in device memory, or, for lists of at most 16 tensors, searched in a
+// copy that travels as a kernel argument (tables.h).  How many workgroups a CU holds at once
+// is throttled with a dummy dynamic-LDS request (see launch_shape): with up to thirteen
+// concurrent streams HBM runs best when only a few tens of KiB per CU are in flight.
 //
 // Arithmetic contract.  Results follow optimi's PyTorch for-loop path
 // (optimi/adam.py:354-396, lion.py:301-338, stableadamw.py:421-472, adan.py:405-469),
@@ -825,7 +826,6 @@ int staged_upload(optimi_group* g, void* dst, const void* src, size_t bytes, hip
   return 0;
 }
 
-int check_ptrs(int n_tensors, const void* const* list) { return (n_tensors > 0 && list == nullptr) ? OPTIMI_ERR_NULL : 0; }
 
 // A list whose arrays add up to at most this many bytes stays in the 256 MB last-level cache
 // from one optimizer step to the next (measured: cached loads beat `nt` loads up to 270 MB of

@@ -24,9 +24,10 @@ def _addr(t):
 class HipRun(ForLoopRun):
     """``multi=True``: whole-list entry points (one launch); False: per-tensor entry points."""
 
-    def __init__(self, name, params, *, multi=True, **kw):
+    def __init__(self, name, params, *, multi=True, cold=False, **kw):
         super().__init__(name, params, **kw)
         self.multi = multi
+        self.cold = cold  # pass OPTIMI_COLD to the whole-list entry points
         self.group = cabi.Group()
         self.entry = "adam" if name == "adamw" else name
 
@@ -64,6 +65,8 @@ class HipRun(ForLoopRun):
             return
         dt = DT[ps[0].dtype]
         if self.multi and not self.gradient_release:
+            if self.cold:
+                scalars = scalars[:-1] + (scalars[-1] | cabi.COLD,)
             cols = [cabi.ptr_array(_addr(p) for p in ps), cabi.ptr_array(_addr(g) for g in grads)]
             cols += [cabi.ptr_array(_addr(s[k]) for s in sts) for k in STATE_ORDER[self.name]]
             cols.append(cabi.ptr_array(_addr(s["kahan_comp"]) for s in sts))
