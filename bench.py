@@ -71,7 +71,16 @@ def workloads():
         "radam_bf16_kahan_llama7b": ("RAdam", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2, decouple_wd=True), "bfloat16", l7, 18),
         # as Adam; every k-th step also reads and writes the slow weights (4 more bytes per param on that step)
         "ranger_bf16_kahan_llama7b": ("Ranger", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2, k=6, alpha=0.5), "bfloat16", l7, 18),
+        # the same list with the embeddings and the norm weights kept in fp32 (FP32_TENSORS): one launch over both
+        # dtypes; 18 bytes per bf16 parameter, 28 per fp32 one
+        "adamw_bf16_kahan_fp32_embeddings_norms_llama7b": ("AdamW", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2), "bfloat16", l7, 18),
     }
+
+
+# workload -> which tensors of its list are fp32 instead of the workload's dtype
+FP32_TENSORS = {
+    "adamw_bf16_kahan_fp32_embeddings_norms_llama7b": lambda shape: len(shape) == 1 or shape[0] == 32000,
+}
 
 
 # HBM bytes per step read off the hardware counters in a separate profiler run (rocprofv3 --pmc
@@ -89,7 +98,8 @@ MEASURED_TRAFFIC = {
 # the benchmark configurations reported under "extra" next to the headline workload
 EXTRA_WORKLOADS = [
     "adamw_fp32_mlp", "adamw_bf16_kahan_declr_llama1b", "lion_bf16_kahan_llama7b", "stableadamw_bf16_kahan_llama7b",
-    "adan_bf16_kahan_llama7b", "adamw_bf16_kahan_release_llama7b", "adamw_bf16_kahan_release_stress10k",
+    "adan_bf16_kahan_llama7b", "adamw_bf16_kahan_fp32_embeddings_norms_llama7b", "adamw_bf16_kahan_release_llama7b",
+    "adamw_bf16_kahan_release_stress10k",
 ]
 RELEASE_WORKLOADS = ("adamw_bf16_kahan_release_stress10k", "adamw_bf16_kahan_release_llama7b")
 
@@ -105,13 +115,14 @@ def make_tensors(shapes, dtype, device, seed, std, ones_for_1d=False):
     import torch
 
     gen = torch.Generator(device=device).manual_seed(seed)
+    dtypes = dtype if isinstance(dtype, (list, tuple)) else [dtype] * len(shapes)
     out = []
-    for s in shapes:
+    for s, dt in zip(shapes, dtypes):
         if ones_for_1d and len(s) == 1:
-            out.append(torch.ones(s, dtype=dtype, device=device))
+            out.append(torch.ones(s, dtype=dt, device=device))
         else:
             t = torch.empty(s, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
-            out.append(t.to(dtype))
+            out.append(t.to(dt))
             del t
     return out
 
@@ -267,9 +278,14 @@ def list_bench(workload, args, steps, warmup):
     cls_name, kwargs, dtype_name, shapes, bytes_per_param = workloads()[workload]
     dtype = getattr(torch, dtype_name)
     n_params = sum(numel(s) for s in shapes)
+    is_fp32 = FP32_TENSORS.get(workload)
+    dtypes = [torch.float32 if (is_fp32 and is_fp32(s)) else dtype for s in shapes]
+    n_fp32 = sum(numel(s) for s, dt in zip(shapes, dtypes) if dt == torch.float32) if is_fp32 else 0
+    if is_fp32:  # the average over the list: 28 bytes per fp32 parameter (four arrays read, three written)
+        bytes_per_param = (bytes_per_param * (n_params - n_fp32) + 28 * n_fp32) / n_params
 
-    params = [torch.nn.Parameter(p) for p in make_tensors(shapes, dtype, device, 0, 0.02, ones_for_1d=True)]
-    grad_sets = [make_tensors(shapes, dtype, device, 100 + i, 1e-3) for i in range(max(1, args.grad_sets))]
+    params = [torch.nn.Parameter(p) for p in make_tensors(shapes, dtypes, device, 0, 0.02, ones_for_1d=True)]
+    grad_sets = [make_tensors(shapes, dtypes, device, 100 + i, 1e-3) for i in range(max(1, args.grad_sets))]
     opt = getattr(optimi_amd, cls_name)(params, **kwargs)
 
     def one_step(i):
@@ -317,6 +333,7 @@ def list_bench(workload, args, steps, warmup):
         "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype],
         "data": "synthetic",
         "config": {"workload": workload, "optimizer": cls_name, "n_tensors": len(shapes), "n_params": n_params,
+                   **({"n_params_fp32": n_fp32} if is_fp32 else {}),
                    "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()},
                    "grad_sets": len(grad_sets)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -331,7 +348,8 @@ def list_bench(workload, args, steps, warmup):
         out["roofline"]["traffic_note"] = "no hardware-counter profile is kept for this workload"
     del opt, params, grad_sets
     torch.cuda.empty_cache()
-    return out, (cls_name, kwargs, dtype, shapes)
+    # the CPU baseline is timed for lists of one dtype only
+    return out, (None if is_fp32 else (cls_name, kwargs, dtype, shapes))
 
 
 def run_workload(workload, args, steps, warmup):

@@ -157,6 +157,53 @@ int optimi_hip_ranger_multi(optimi_group* group, int n_tensors, void* const* par
                             double alpha, uint32_t flags, optimi_stream_t stream);
 
 /* ---------------------------------------------------------------------------------
+ * Whole-list steps over a list of mixed dtypes: the same steps, still one launch, for a
+ * parameter group that holds fp32 tensors beside tensors of one 16-bit dtype (a model kept
+ * in bf16 whose embeddings or norms stay fp32).  The reference's launchers loop over the
+ * tensors of a group whatever their dtypes (optimi/adam.py:551-583 and the same loop in
+ * lion.py, stableadamw.py, adan.py, sgd.py, radam.py, ranger.py); these entry points keep such a
+ * group in one launch.  They differ from their `_multi` namesakes in one argument: `dtype`
+ * is an array with every tensor's own dtype.  bf16 and fp16 in one list is OPTIMI_ERR_DTYPE.
+ * OPTIMI_KAHAN applies to the 16-bit tensors only; kahan_comp[i] of an fp32 tensor is ignored
+ * and may be NULL.  Every tensor gets the bits its dtype's `_multi` call would give it.  A
+ * list that turns out to hold one dtype is stepped exactly as by `_multi`.
+ * ------------------------------------------------------------------------------- */
+int optimi_hip_adam_multi_mixed(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                                void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                                const int64_t* numel, const int* dtype, double lr, double beta1_comp, double beta2_hat,
+                                double beta2_comp, double weight_decay, double eps, uint32_t flags,
+                                optimi_stream_t stream);
+int optimi_hip_lion_multi_mixed(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                                void* const* exp_avg, void* const* kahan_comp, const int64_t* numel, const int* dtype,
+                                double lr, double beta1_comp, double beta2_comp, double weight_decay, uint32_t flags,
+                                optimi_stream_t stream);
+int optimi_hip_stableadamw_multi_mixed(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                                       void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                                       const int64_t* numel, const int* dtype, double lr, double beta1_comp,
+                                       double beta2_hat, double beta2_comp, double weight_decay, double eps,
+                                       double max_lr, uint32_t flags, optimi_stream_t stream);
+int optimi_hip_adan_multi_mixed(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                                void* const* exp_avg, void* const* exp_avg_diff, void* const* exp_avg_sq,
+                                void* const* prev_grad, void* const* kahan_comp, const int64_t* numel, const int* dtype,
+                                double lr, double beta1_comp, double beta2, double beta2_comp, double beta3_hat,
+                                double beta3_comp, double eps, double weight_decay, uint32_t flags,
+                                optimi_stream_t stream);
+int optimi_hip_sgd_multi_mixed(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                               void* const* exp_avg, void* const* kahan_comp, const int64_t* numel, const int* dtype,
+                               double lr, double momentum, double weight_decay, uint32_t flags,
+                               optimi_stream_t stream);
+int optimi_hip_radam_multi_mixed(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                                 void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                                 const int64_t* numel, const int* dtype, double lr, double beta1_comp, double beta2_hat,
+                                 double beta2_comp, double weight_decay, double eps, double rect, uint32_t flags,
+                                 optimi_stream_t stream);
+int optimi_hip_ranger_multi_mixed(optimi_group* group, int n_tensors, void* const* param, const void* const* grad,
+                                  void* const* exp_avg, void* const* exp_avg_sq, void* const* la_param,
+                                  void* const* kahan_comp, const int64_t* numel, const int* dtype, double lr,
+                                  double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay,
+                                  double eps, double rect, double alpha, uint32_t flags, optimi_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
  * Per-tensor steps for gradient release: pointers travel as kernel arguments, no table.
  * ------------------------------------------------------------------------------- */
 
@@ -224,6 +271,11 @@ int optimi_hip_ranger_single(void* param, const void* grad, void* exp_avg, void*
  * the practical bandwidth ceiling and to scale hardware byte counters.
  * ------------------------------------------------------------------------------- */
 int optimi_hip_copy_probe(void* dst, const void* src, int64_t bytes, optimi_stream_t stream);
+
+/* Measurement aid (no counterpart in the reference): the number of kernels this library has
+ * launched in this process so far, every entry point and every thread counted.  Tests and
+ * benchmarks take differences of it to see how many launches a step costs. */
+int64_t optimi_hip_launch_count(void);
 
 #ifdef __cplusplus
 }

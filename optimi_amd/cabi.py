@@ -18,6 +18,7 @@ KAHAN, UPDATE, DECOUPLE_WD, ADAM_WD, DECOUPLE_LR, DAMPENING, RECTIFY, LOOKAHEAD,
 
 _p, _pp, _i, _i64, _u32, _d = C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_int64, C.c_uint32, C.c_double
 _i64p = C.POINTER(C.c_int64)
+_ip = C.POINTER(C.c_int)
 
 PROTOTYPES = {
     "optimi_hip_error_string": (C.c_char_p, [_i]),
@@ -32,6 +33,13 @@ PROTOTYPES = {
     "optimi_hip_sgd_multi": (_i, [_p, _i, _pp, _pp, _pp, _pp, _i64p, _i, _d, _d, _d, _u32, _p]),
     "optimi_hip_radam_multi": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _i64p, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_ranger_multi": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _pp, _i64p, _i, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_adam_multi_mixed": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _i64p, _ip, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_lion_multi_mixed": (_i, [_p, _i, _pp, _pp, _pp, _pp, _i64p, _ip, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_stableadamw_multi_mixed": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _i64p, _ip, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_adan_multi_mixed": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _pp, _pp, _i64p, _ip, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_sgd_multi_mixed": (_i, [_p, _i, _pp, _pp, _pp, _pp, _i64p, _ip, _d, _d, _d, _u32, _p]),
+    "optimi_hip_radam_multi_mixed": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _i64p, _ip, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
+    "optimi_hip_ranger_multi_mixed": (_i, [_p, _i, _pp, _pp, _pp, _pp, _pp, _pp, _i64p, _ip, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_adam_single": (_i, [_p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_lion_single": (_i, [_p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_stableadamw_single": (_i, [_p, _p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
@@ -41,6 +49,7 @@ PROTOTYPES = {
     "optimi_hip_radam_single": (_i, [_p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_ranger_single": (_i, [_p, _p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_copy_probe": (_i, [_p, _p, _i64, _p]),
+    "optimi_hip_launch_count": (_i64, []),
 }
 
 _lib = None

@@ -25,6 +25,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdlib>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -56,7 +57,7 @@ constexpr int kSub = kChunkBytes / (kThreads * kUnroll * 16);  // workgroups per
 static_assert(kSub >= 1 && kSub * kThreads * kUnroll * 16 == kChunkBytes, "workgroup tile must divide the chunk");
 static_assert(kThreads % 64 == 0 && kThreads <= 1024, "whole wavefronts");
 constexpr int kReduceThreads = 1024;      // lanes of the per-tensor finalize workgroup
-constexpr int kAbiVersion = 1001;
+constexpr int kAbiVersion = 1002;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -227,6 +228,7 @@ struct AdamScalars {
 template <class DT_, bool KAHAN, bool UPDATE, int WD, int TAIL>
 struct AdamTailOp {
   using DT = DT_;
+  using F32Partner = AdamTailOp<F32, false, UPDATE, WD, TAIL>;  // the same step on an fp32 tensor of a mixed list
   using Scalars = AdamScalars;
   static constexpr int kArrays = 5;
   static constexpr uint32_t kLoad = UPDATE ? (bit(0) | bit(1) | bit(2) | bit(3) | (KAHAN ? bit(4) : 0)) : (bit(1) | bit(2) | bit(3));
@@ -275,6 +277,7 @@ struct RangerScalars {
 template <class DT_, bool KAHAN, bool UPDATE, int WD, int TAIL, bool LA>
 struct RangerOp {
   using DT = DT_;
+  using F32Partner = RangerOp<F32, false, UPDATE, WD, TAIL, LA>;
   using Scalars = RangerScalars;
   using Inner = AdamTailOp<DT_, KAHAN, UPDATE, WD, TAIL>;
   static constexpr int kArrays = 6;
@@ -314,6 +317,7 @@ struct SgdScalars {
 template <class DT_, bool KAHAN, bool UPDATE, int WD, int MOM>
 struct SgdOp {
   using DT = DT_;
+  using F32Partner = SgdOp<F32, false, UPDATE, WD, MOM>;
   using Scalars = SgdScalars;
   static constexpr int kArrays = 4;
   static constexpr uint32_t kLoad = bit(1) | (MOM ? bit(2) : 0) | (UPDATE ? (bit(0) | (KAHAN ? bit(3) : 0)) : 0);
@@ -357,6 +361,7 @@ struct LionScalars {
 template <class DT_, bool KAHAN, bool UPDATE, int WD>
 struct LionOp {
   using DT = DT_;
+  using F32Partner = LionOp<F32, false, UPDATE, WD>;
   using Scalars = LionScalars;
   static constexpr int kArrays = 4;
   static constexpr uint32_t kLoad = UPDATE ? (bit(0) | bit(1) | bit(2) | (KAHAN ? bit(3) : 0)) : (bit(1) | bit(2));
@@ -398,6 +403,7 @@ struct StableP1Scalars {
 template <class DT_, bool UPDATE>
 struct StablePass1Op {
   using DT = DT_;
+  using F32Partner = StablePass1Op<F32, UPDATE>;
   using Scalars = StableP1Scalars;
   static constexpr int kArrays = 5;
   static constexpr uint32_t kLoad = bit(1) | bit(2) | bit(3);
@@ -429,6 +435,7 @@ struct StableP2Scalars {
 template <class DT_, bool KAHAN, int WD>
 struct StablePass2Op {
   using DT = DT_;
+  using F32Partner = StablePass2Op<F32, false, WD>;
   using Scalars = StableP2Scalars;
   static constexpr int kArrays = 5;
   static constexpr uint32_t kLoad = bit(0) | bit(2) | bit(3) | (KAHAN ? bit(4) : 0);
@@ -466,6 +473,7 @@ struct AdanScalars {
 template <class DT_, bool KAHAN, bool UPDATE, int WD>
 struct AdanOp {
   using DT = DT_;
+  using F32Partner = AdanOp<F32, false, UPDATE, WD>;
   using Scalars = AdanScalars;
   static constexpr int kArrays = 7;
   static constexpr uint32_t kState = bit(2) | bit(3) | bit(4) | bit(5);
@@ -604,24 +612,17 @@ __device__ __forceinline__ void one_element(const TensorEntry& e, int64_t i, con
     if (Op::kStore & bit(a)) DT::store1(e.ptr[a], i, x[a].x);
 }
 
-// MULTI: the tensor table and the chunk map are in device memory.  Otherwise the table travels
-// as the kernel argument `few` (one tensor for the per-tensor entry points, up to kFew for
-// short lists) and the workgroup searches it.
-template <class Op, bool MULTI>
-__global__ void __launch_bounds__(kThreads)
-step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, const FewTable few,
-            typename Op::Scalars s, double* __restrict__ partials) {
+// The work of one workgroup: the tile `sub` of chunk `chunk_id`, which belongs to tensor `tensor`
+// (entry `e`).  `s` is the workgroup's own copy of the launch scalars.
+template <class Op>
+__device__ __forceinline__ void tile_step(const TensorEntry& e, int tensor, int64_t chunk_id, int sub,
+                                          typename Op::Scalars s, double* __restrict__ partials) {
   using DT = typename Op::DT;
   constexpr int V = DT::kVec;
   constexpr int A = Op::kArrays;
   constexpr int64_t kChunk = chunk_elems<DT>();
   constexpr int64_t kTile = (int64_t)kThreads * kUnroll * V;  // elements one workgroup covers
 
-  const int64_t chunk_id = blockIdx.x / kSub;
-  const int sub = blockIdx.x % kSub;
-  // a table of one (the per-tensor entry points) needs no search
-  const int tensor = MULTI ? chunk_map[chunk_id] : (few.n == 1 ? 0 : optimi_tables::few_lookup(few, chunk_id));
-  const TensorEntry& e = MULTI ? table[tensor] : few.e[tensor];
   const int64_t base = optimi_tables::tile_base(chunk_id, sub, e.first_chunk, kChunk, kTile);
   const int64_t remain = e.numel - base;  // <= 0 for tiles past the end of the tensor's last chunk
   const bool vec_ok = (e.flags & optimi_tables::kEntryVec) != 0;
@@ -672,10 +673,42 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
   }
 }
 
+// MULTI: the tensor table and the chunk map are in device memory.  Otherwise the table travels
+// as the kernel argument `few` (one tensor for the per-tensor entry points, up to kFew for
+// short lists) and the workgroup searches it.
+template <class Op, bool MULTI>
+__global__ void __launch_bounds__(kThreads)
+step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, const FewTable few,
+            typename Op::Scalars s, double* __restrict__ partials) {
+  const int64_t chunk_id = blockIdx.x / kSub;
+  const int sub = blockIdx.x % kSub;
+  // a table of one (the per-tensor entry points) needs no search
+  const int tensor = MULTI ? chunk_map[chunk_id] : (few.n == 1 ? 0 : optimi_tables::few_lookup(few, chunk_id));
+  const TensorEntry& e = MULTI ? table[tensor] : few.e[tensor];
+  tile_step<Op>(e, tensor, chunk_id, sub, s, partials);
+}
+
+// A list that holds fp32 tensors beside tensors of one 16-bit dtype (a model kept in bf16 whose
+// embeddings or norms stay fp32): every workgroup looks its tensor up as above and runs that
+// dtype's step on its tile, with that dtype's scalars.  Chunks are kChunkBytes per array for
+// both, so the grid does not care which is which.
+template <class OpLow, class OpF32>
+__global__ void __launch_bounds__(kThreads)
+mixed_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, typename OpLow::Scalars s_low,
+             typename OpF32::Scalars s_f32, double* __restrict__ partials) {
+  const int64_t chunk_id = blockIdx.x / kSub;
+  const int sub = blockIdx.x % kSub;
+  const int tensor = chunk_map[chunk_id];
+  const TensorEntry& e = table[tensor];
+  if (e.flags & optimi_tables::kEntryF32) tile_step<OpF32>(e, tensor, chunk_id, sub, s_f32, partials);
+  else tile_step<OpLow>(e, tensor, chunk_id, sub, s_low, partials);
+}
+
 // StableAdamW: one workgroup per tensor turns that tensor's chunk partials into its clipped
 // learning rate and decay factor (optimi/stableadamw.py:447-458), in double like the Python
 // scalars of the reference.  The mean and its square root are rounded to the tensor dtype,
-// as torch's mean()/sqrt() on a tensor of that dtype are.
+// as torch's mean()/sqrt() on a tensor of that dtype are.  `DT` is the dtype of the list's
+// tensors that are not marked fp32 in their entry.
 struct FinalizeArgs {
   double lr, weight_decay, max_lr;
   uint32_t decouple_lr;
@@ -685,10 +718,11 @@ template <class DT, bool MULTI>
 __global__ void __launch_bounds__(kReduceThreads)
 stable_finalize_kernel(const TensorEntry* __restrict__ table, const FewTable few, const double* __restrict__ partials,
                        TensorScalars* __restrict__ out, FinalizeArgs a) {
-  constexpr int64_t kChunk = chunk_elems<DT>();
   const TensorEntry& e = MULTI ? table[blockIdx.x] : few.e[blockIdx.x];
+  const bool f32 = (e.flags & optimi_tables::kEntryF32) != 0;
+  const int64_t chunk = f32 ? chunk_elems<F32>() : chunk_elems<DT>();
   const int64_t first = e.first_chunk * kSub;  // one partial per workgroup of pass 1
-  const int64_t count = (e.numel + kChunk - 1) / kChunk * kSub;
+  const int64_t count = (e.numel + chunk - 1) / chunk * kSub;
   // four independent accumulators keep several loads in flight; the order is fixed, so the sum is
   // the same on every run
   double v0 = 0.0, v1 = 0.0, v2 = 0.0, v3 = 0.0;
@@ -706,8 +740,10 @@ stable_finalize_kernel(const TensorEntry* __restrict__ table, const FewTable few
   if (threadIdx.x == 0) {
     double lr = a.lr;
     if (e.numel > 0) {
-      float ms = DT::R2(splat((float)total / (float)e.numel)).x;
-      float rms = DT::R2(splat(sqrtf(ms))).x;
+      float ms = (float)total / (float)e.numel;
+      if (!f32) ms = DT::R2(splat(ms)).x;
+      float rms = sqrtf(ms);
+      if (!f32) rms = DT::R2(splat(rms)).x;
       double r = (double)rms;
       lr = lr / (r > 1.0 ? r : 1.0);
     }
@@ -791,8 +827,7 @@ struct optimi_group {
   DeviceBuf table, chunk_map, partials, tensor_scalars;
   std::vector<TensorEntry> host_table;   // what the device table holds
   std::vector<int32_t> host_map;         // scratch for building the chunk map
-  std::vector<int64_t> map_numel;        // sizes the device chunk map was built for
-  int64_t map_chunk = 0;
+  std::vector<int64_t> map_first;        // what the device chunk map was built for: every tensor's first chunk, then the chunk count
   StagingSlot ring[4];
   int ring_pos = 0;
   hipEvent_t last_launch = nullptr;
@@ -830,13 +865,10 @@ int staged_upload(optimi_group* g, void* dst, const void* src, size_t bytes, hip
 // A list whose arrays add up to at most this many bytes stays in the 256 MB last-level cache
 // from one optimizer step to the next (measured: cached loads beat `nt` loads up to 270 MB of
 // arrays and lose from 335 MB on).  Such a launch - unless the caller marks it OPTIMI_COLD -
-// uses cached loads and, being short, 21 resident workgroups per CU (16.8 M fp32 parameters in
-// one launch: 83 us -> 78 us).  Per-tensor entry points never take this path: they step one
-// tensor of a larger model, which was last touched a whole backward pass ago (measured on
-// tensors that are cold when revisited: `nt` loads and the table's occupancy are 6-8 % faster
-// there than cached loads or 21 workgroups).
+// uses cached loads.  Per-tensor entry points never take this path: they step one tensor of a
+// larger model, which was last touched a whole backward pass ago (measured on tensors that are
+// cold when revisited: `nt` loads are 6-8 % faster there than cached ones).
 constexpr int64_t kResidentBytes = (int64_t)288 << 20;
-constexpr int kResidentGranules = 6;
 
 // What one list launch works on, as the entry points hand it to the launchers.
 struct ListPlan {
@@ -845,16 +877,38 @@ struct ListPlan {
   int n_tensors = 0;
   int64_t n_chunks = 0;
   bool resident = false;      // the list's arrays fit the last-level cache and were touched recently
+  bool mixed = false;         // fp32 tensors beside 16-bit ones (always through the device tables)
 };
 
 constexpr int64_t kMaxChunks = (int64_t)0x7fffffff / kSub;  // the grid is chunks x kSub workgroups
 
+// The dtypes a mixed list may hold: fp32 and at most one 16-bit dtype.  `*low` becomes the
+// dtype of the tensors that are not fp32 (fp32 if there are none), `*mixed` whether both kinds
+// are present.
+int list_dtypes(int n_tensors, const int* dtypes, int* low, bool* mixed) {
+  if (n_tensors > 0 && !dtypes) return OPTIMI_ERR_NULL;
+  int low_dtype = OPTIMI_F32;
+  bool any_f32 = false;
+  for (int t = 0; t < n_tensors; ++t) {
+    if (!valid_dtype(dtypes[t])) return OPTIMI_ERR_DTYPE;
+    if (dtypes[t] == OPTIMI_F32) any_f32 = true;
+    else if (low_dtype == OPTIMI_F32) low_dtype = dtypes[t];
+    else if (low_dtype != dtypes[t]) return OPTIMI_ERR_DTYPE;  // bf16 and fp16 in one list
+  }
+  *low = low_dtype;
+  *mixed = any_f32 && low_dtype != OPTIMI_F32;
+  return 0;
+}
+
 // Validates the list and gets its tables to where the kernel reads them: into `plan` itself for
-// a list of at most kFew tensors (nothing is uploaded), else into the group's device tables,
-// (re)building the chunk map and tensor table and uploading what changed.
+// a list of at most kFew tensors of one dtype (nothing is uploaded), else into the group's device
+// tables, (re)building the chunk map and tensor table and uploading what changed.
 // `lists[a]` may be nullptr for an array the launch does not touch (`need` has its bit clear).
+// `dtypes`: nullptr when every tensor has `dtype`; else every tensor's own dtype, `dtype` being
+// the 16-bit one among them, and fp32 tensors have no array in `low_precision_only`.
 int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, int n_arrays, uint32_t need,
-              const int64_t* numel, int dtype, uint32_t flags, hipStream_t stream, ListPlan* plan) {
+              uint32_t low_precision_only, const int64_t* numel, const int* dtypes, int dtype, uint32_t flags,
+              hipStream_t stream, ListPlan* plan) {
   if (!g) return OPTIMI_ERR_NULL;
   if (n_tensors < 0) return OPTIMI_ERR_SIZE;
   if (!valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
@@ -862,9 +916,9 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
   HIP_TRY(hipGetDevice(&dev));
   if (dev != g->device) return OPTIMI_ERR_DEVICE;
 
-  const int64_t chunk = chunk_elems_rt(dtype);
   plan->n_tensors = n_tensors;
-  plan->few = n_tensors <= kFew;
+  plan->mixed = dtypes != nullptr;
+  plan->few = n_tensors <= kFew && !plan->mixed;
   std::memset(&plan->table, 0, sizeof(plan->table));
   std::vector<TensorEntry> fresh;
   TensorEntry* entries = plan->table.e;
@@ -877,12 +931,16 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
     entries = fresh.data();
   }
   int64_t n_chunks = 0;
-  int rc = optimi_tables::build_entries(n_tensors, lists, n_arrays, need, numel, dtype, kMaxChunks, entries, &n_chunks);
+  int rc = optimi_tables::build_entries(n_tensors, lists, n_arrays, need, numel, dtypes, dtype, low_precision_only,
+                                        kMaxChunks, entries, &n_chunks);
   if (rc) return rc;
   plan->n_chunks = n_chunks;
-  int64_t total = 0;
-  for (int t = 0; t < n_tensors; ++t) total += numel[t];
-  plan->resident = !(flags & OPTIMI_COLD) && total * elem_bytes(dtype) * popcount(need) <= kResidentBytes;
+  int64_t bytes = 0;
+  for (int t = 0; t < n_tensors; ++t) {
+    const bool f32 = (entries[t].flags & optimi_tables::kEntryF32) != 0;
+    bytes += numel[t] * (f32 ? 4 : 2) * popcount(f32 ? need & ~low_precision_only : need);
+  }
+  plan->resident = !(flags & OPTIMI_COLD) && bytes <= kResidentBytes;
   if (plan->resident)
     for (int t = 0; t < n_tensors; ++t) entries[t].flags |= optimi_tables::kEntryCached;
   if (plan->few) {
@@ -893,22 +951,28 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
   // a group moved to another stream must not overwrite tables a previous launch still reads
   if (g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
 
-  bool same_sizes = g->map_chunk == chunk && g->map_numel.size() == (size_t)n_tensors &&
-                    std::memcmp(g->map_numel.data(), numel, sizeof(int64_t) * (size_t)n_tensors) == 0;
-  if (!same_sizes && n_chunks > 0) {
-    g->map_chunk = 0;  // the cached map is void until the new one is on its way
+  // the chunk map is a function of where every tensor's chunks start and of how many there are
+  bool same_map = g->map_first.size() == (size_t)n_tensors + 1 && g->map_first[(size_t)n_tensors] == n_chunks;
+  for (int t = 0; same_map && t < n_tensors; ++t) same_map = g->map_first[(size_t)t] == fresh[(size_t)t].first_chunk;
+  if (!same_map && n_chunks > 0) {
+    g->map_first.clear();  // the cached map is void until the new one is on its way
     try {
       g->host_map.resize((size_t)n_chunks);
-      g->map_numel.assign(numel, numel + n_tensors);
     } catch (const std::bad_alloc&) {
       return OPTIMI_ERR_NOMEM;
     }
-    optimi_tables::build_chunk_map(fresh.data(), n_tensors, chunk, g->host_map.data());
+    optimi_tables::build_chunk_map(fresh.data(), n_tensors, g->host_map.data());
     rc = g->chunk_map.reserve(sizeof(int32_t) * (size_t)n_chunks);
     if (rc) return rc;
     rc = staged_upload(g, g->chunk_map.ptr, g->host_map.data(), sizeof(int32_t) * (size_t)n_chunks, stream);
     if (rc) return rc;
-    g->map_chunk = chunk;
+    try {
+      g->map_first.resize((size_t)n_tensors + 1);
+    } catch (const std::bad_alloc&) {
+      return OPTIMI_ERR_NOMEM;
+    }
+    for (int t = 0; t < n_tensors; ++t) g->map_first[(size_t)t] = fresh[(size_t)t].first_chunk;
+    g->map_first[(size_t)n_tensors] = n_chunks;
   }
 
   bool same_table = g->host_table.size() == fresh.size() &&
@@ -956,10 +1020,13 @@ int finish_list(optimi_group* g, const ListPlan& plan, hipStream_t stream) {
 // workgroups; reachable occupancies are therefore 32, 25, 21, 18, 16, 14, 12, 11, 10, 9, 8, ...
 // The table holds the measured optimum in granules on MI355X with the write-through tile stores
 // (7B-parameter lists; 5 streams = StableAdamW pass 1 and accumulate-only Adam, 6 = pass 2,
-// 7 = Lion / SGD, 9 = Adam with Kahan, 13 = Adan; entries in between are interpolated).  fp32
-// lists with 7 streams do best at 12 workgroups instead of 11.  16-bit list launches of fewer
-// than kLongLaunch workgroups (the Llama-1B-shaped list) do best one granule lower, i.e. with
-// one more workgroup resident.  OPTIMI_HIP_WAVES overrides the number of wavefronts
+// 7 = Lion / SGD and fp32 Adam, 9 = Adam with Kahan, 13 = Adan; entries in between are
+// interpolated).  fp32 Adan (11 streams) does best at 17 granules, 7 workgroups (a Llama-1B-shaped
+// list: 8.12 ms at 16, 7.98 ms at 17 and 18).  16-bit list launches of fewer than kLongLaunch
+// workgroups (the Llama-1B-shaped list) do best one granule lower, i.e. with one more workgroup
+// resident.  Lists that live in the last-level cache follow the same table (16.8 M parameters:
+// fp32 AdamW 68.9 us at 6 granules, 67.5 us at 10 and 11; bf16 AdamW 48.7 us at 6, 47.0 us at 12;
+// fp32 Adan 131 us at 6, 120 us at 14).  OPTIMI_HIP_WAVES overrides the number of wavefronts
 // per CU for every kernel (nearest reachable count at or above it; 0 = no throttle); read once.
 constexpr int kLdsGranule = 1280, kLdsGranules = 128;
 constexpr int kMaxStreams = 2 * kMaxArrays;
@@ -989,15 +1056,14 @@ struct LaunchShape {
 // launches under kLongLaunch), 9 granules instead of 8 for 5 and 6 streams (measured on
 // per-tensor launches over tensors that are cold when revisited, 4 M to 45 M elements).
 template <class Op>
-LaunchShape launch_shape(int64_t workgroups, bool resident, bool few) {
+LaunchShape launch_shape(int64_t workgroups, bool few) {
   constexpr int streams = (popcount(Op::kLoad) + popcount(Op::kStore)) * kUnroll;
   constexpr bool f32 = std::is_same<typename Op::DT, F32>::value;
   LaunchShape shape;
   int granules = kBestGranules[streams < kMaxStreams ? streams : kMaxStreams];
-  if (f32 && streams == 7) granules = 10;
+  if (f32 && streams == 11) granules = 17;
   if (!few && !f32 && streams >= 7 && workgroups < kLongLaunch) granules -= 1;
   if (few && (streams == 5 || streams == 6)) granules = 9;
-  if (resident) granules = kResidentGranules;
 #ifdef OPTIMI_TUNING
   if (const char* env = std::getenv("OPTIMI_HIP_LDS")) {  // raw request, tuning builds only
     shape.lds = (unsigned)std::strtol(env, nullptr, 10);
@@ -1023,11 +1089,22 @@ LaunchShape launch_shape(int64_t workgroups, bool resident, bool few) {
 
 const FewTable kNoTable = {};
 
+std::atomic<int64_t> kernel_launches{0};  // every kernel this library has launched in this process
+
+// `s_f32`: the same scalars formed for fp32 tensors; read only when the plan is a mixed list.
 template <class Op>
 void launch_list(optimi_group* g, const ListPlan& plan, const typename Op::Scalars& s, hipStream_t stream,
-                 double* partials = nullptr) {
+                 double* partials = nullptr, const typename Op::Scalars* s_f32 = nullptr) {
   const int64_t workgroups = plan.n_chunks * kSub;
-  const LaunchShape shape = launch_shape<Op>(workgroups, plan.resident, plan.few);
+  const LaunchShape shape = launch_shape<Op>(workgroups, plan.few);
+  ++kernel_launches;
+  if constexpr (!std::is_same<typename Op::DT, F32>::value) {
+    if (plan.mixed) {
+      mixed_kernel<Op, typename Op::F32Partner><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
+          (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, s, *s_f32, partials);
+      return;
+    }
+  }
   if (plan.few)
     step_kernel<Op, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
         nullptr, nullptr, plan.table, s, partials);
@@ -1048,7 +1125,8 @@ template <class Op>
 void launch_single(const TensorEntry& e, const typename Op::Scalars& s, double* partials, hipStream_t stream) {
   const int64_t chunk = chunk_elems<typename Op::DT>();
   const int64_t workgroups = (e.numel + chunk - 1) / chunk * kSub;
-  const LaunchShape shape = launch_shape<Op>(workgroups, false, true);
+  const LaunchShape shape = launch_shape<Op>(workgroups, true);
+  ++kernel_launches;
   step_kernel<Op, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
       nullptr, nullptr, table_of_one(e), s, partials);
 }
@@ -1111,7 +1189,7 @@ int single_entry(TensorEntry& e, const void* const* ptrs, int n_arrays, uint32_t
   if (numel > chunk_elems_rt(dtype) * ((int64_t)0x7fffffff / kSub)) return OPTIMI_ERR_SIZE;
   std::memset(&e, 0, sizeof(e));
   e.numel = numel;
-  e.flags = optimi_tables::kEntryVec;
+  e.flags = optimi_tables::kEntryVec | (dtype == OPTIMI_F32 ? optimi_tables::kEntryF32 : 0u);
   const int eb = elem_bytes(dtype);
   for (int a = 0; a < n_arrays; ++a) {
     if (!(need & bit(a))) continue;
@@ -1258,8 +1336,9 @@ int stable_run(const ListPlan* plan, optimi_group* g, const TensorEntry& single,
   const bool update = (flags & OPTIMI_UPDATE) != 0;
   const bool kahan = kahan_on(dtype, flags);
   StableP1Scalars s1 = stable_p1_scalars(dtype, beta1_comp, beta2_hat, beta2_comp, eps);
+  const StableP1Scalars s1_f32 = stable_p1_scalars(OPTIMI_F32, beta1_comp, beta2_hat, beta2_comp, eps);
   if (!update) {
-    if (plan) launch_list<StablePass1Op<DT, false>>(g, *plan, s1, stream);
+    if (plan) launch_list<StablePass1Op<DT, false>>(g, *plan, s1, stream, nullptr, &s1_f32);
     else launch_single<StablePass1Op<DT, false>>(single, s1, nullptr, stream);
     return 0;
   }
@@ -1273,19 +1352,22 @@ int stable_run(const ListPlan* plan, optimi_group* g, const TensorEntry& single,
   s2.eps_d = Sd(eps, dtype);
   s2.neg_lr = 0.0f;
   s2.wd = 0.0f;
+  StableP2Scalars s2_f32 = s2;
+  s2_f32.eps_d = Sd(eps, OPTIMI_F32);
   const bool wd = weight_decay != 0;
+  ++kernel_launches;  // the finalize kernel below
   if (plan) {
-    launch_list<StablePass1Op<DT, true>>(g, *plan, s1, stream, scratch.partials);
+    launch_list<StablePass1Op<DT, true>>(g, *plan, s1, stream, scratch.partials, &s1_f32);
     if (plan->few)
       stable_finalize_kernel<DT, false><<<dim3((unsigned)plan->n_tensors), dim3(kReduceThreads), 0, stream>>>(
           nullptr, plan->table, scratch.partials, scratch.tensor_scalars, fa);
     else
       stable_finalize_kernel<DT, true><<<dim3((unsigned)plan->n_tensors), dim3(kReduceThreads), 0, stream>>>(
           (const TensorEntry*)g->table.ptr, kNoTable, scratch.partials, scratch.tensor_scalars, fa);
-    if (kahan && wd) launch_list<StablePass2Op<DT, true, 1>>(g, *plan, s2, stream);
-    else if (kahan) launch_list<StablePass2Op<DT, true, 0>>(g, *plan, s2, stream);
-    else if (wd) launch_list<StablePass2Op<DT, false, 1>>(g, *plan, s2, stream);
-    else launch_list<StablePass2Op<DT, false, 0>>(g, *plan, s2, stream);
+    if (kahan && wd) launch_list<StablePass2Op<DT, true, 1>>(g, *plan, s2, stream, nullptr, &s2_f32);
+    else if (kahan) launch_list<StablePass2Op<DT, true, 0>>(g, *plan, s2, stream, nullptr, &s2_f32);
+    else if (wd) launch_list<StablePass2Op<DT, false, 1>>(g, *plan, s2, stream, nullptr, &s2_f32);
+    else launch_list<StablePass2Op<DT, false, 0>>(g, *plan, s2, stream, nullptr, &s2_f32);
   } else {
     launch_single<StablePass1Op<DT, true>>(single, s1, scratch.partials, stream);
     stable_finalize_kernel<DT, false><<<dim3(1), dim3(kReduceThreads), 0, stream>>>(
@@ -1357,6 +1439,188 @@ int device_scratch(void** out) {
   return 0;
 }
 
+
+// ---- whole-list steps ------------------------------------------------------------------------
+// One function per optimizer behind both of its list entry points.  `dtypes` is nullptr for a
+// list of one dtype (`dtype`); for a mixed list it holds every tensor's dtype.
+
+// Sorts out the dtype arguments of a list call: afterwards `*dtype` is the dtype of the list's
+// 16-bit tensors (or fp32) and `*dtypes` is null unless fp32 and 16-bit tensors are both there.
+int resolve_dtypes(int n_tensors, const int** dtypes, int* dtype) {
+  if (!*dtypes) return valid_dtype(*dtype) ? 0 : OPTIMI_ERR_DTYPE;
+  if (n_tensors < 0) return OPTIMI_ERR_SIZE;
+  bool mixed = false;
+  int rc = list_dtypes(n_tensors, *dtypes, dtype, &mixed);
+  if (rc) return rc;
+  if (!mixed) *dtypes = nullptr;
+  return 0;
+}
+
+int adam_list(optimi_group* g, int n_tensors, void* const* param, const void* const* grad, void* const* exp_avg,
+              void* const* exp_avg_sq, void* const* kahan_comp, const int64_t* numel, const int* dtypes, int dtype,
+              double lr, double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay, double eps,
+              uint32_t flags, hipStream_t stream) {
+  if (!g) return OPTIMI_ERR_NULL;
+  int rc = resolve_dtypes(n_tensors, &dtypes, &dtype);
+  if (rc) return rc;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
+                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
+  ListPlan plan;
+  rc = plan_list(g, n_tensors, lists, 5, adam_need(kahan, update), bit(4), numel, dtypes, dtype, flags, stream, &plan);
+  if (rc) return rc;
+  if (plan.n_chunks == 0) return 0;
+  const AdamScalars s = adam_scalars(dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  const AdamScalars s_f32 = adam_scalars(OPTIMI_F32, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  dispatch<AdamOp, 3>(dtype, kahan, update, adam_wd_mode(weight_decay, flags),
+                      [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream, nullptr, &s_f32); });
+  return finish_list(g, plan, stream);
+}
+
+int lion_list(optimi_group* g, int n_tensors, void* const* param, const void* const* grad, void* const* exp_avg,
+              void* const* kahan_comp, const int64_t* numel, const int* dtypes, int dtype, double lr, double beta1_comp,
+              double beta2_comp, double weight_decay, uint32_t flags, hipStream_t stream) {
+  if (!g) return OPTIMI_ERR_NULL;
+  int rc = resolve_dtypes(n_tensors, &dtypes, &dtype);
+  if (rc) return rc;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const void* const* lists[4] = {(const void* const*)param, grad, (const void* const*)exp_avg,
+                                 (const void* const*)kahan_comp};
+  ListPlan plan;
+  rc = plan_list(g, n_tensors, lists, 4, lion_need(kahan, update), bit(3), numel, dtypes, dtype, flags, stream, &plan);
+  if (rc) return rc;
+  if (plan.n_chunks == 0) return 0;
+  const LionScalars s = lion_scalars(dtype, lr, beta1_comp, beta2_comp, weight_decay);
+  const LionScalars s_f32 = lion_scalars(OPTIMI_F32, lr, beta1_comp, beta2_comp, weight_decay);
+  dispatch<LionOp, 2>(dtype, kahan, update, lion_wd_mode(weight_decay, flags),
+                      [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream, nullptr, &s_f32); });
+  return finish_list(g, plan, stream);
+}
+
+int stableadamw_list(optimi_group* g, int n_tensors, void* const* param, const void* const* grad, void* const* exp_avg,
+                     void* const* exp_avg_sq, void* const* kahan_comp, const int64_t* numel, const int* dtypes, int dtype,
+                     double lr, double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay, double eps,
+                     double max_lr, uint32_t flags, hipStream_t stream) {
+  if (!g) return OPTIMI_ERR_NULL;
+  if ((flags & OPTIMI_DECOUPLE_LR) && weight_decay != 0 && !(max_lr > 0)) return OPTIMI_ERR_ARG;
+  int rc = resolve_dtypes(n_tensors, &dtypes, &dtype);
+  if (rc) return rc;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
+                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
+  ListPlan plan;
+  rc = plan_list(g, n_tensors, lists, 5, adam_need(kahan, update), bit(4), numel, dtypes, dtype, flags, stream, &plan);
+  if (rc) return rc;
+  if (plan.n_chunks == 0) return 0;
+  // the reduction scratch is the group's: a previous launch on another stream may still read it
+  if (plan.few && g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
+  TensorEntry none;
+  std::memset(&none, 0, sizeof(none));
+  rc = dtype == OPTIMI_BF16
+           ? stable_group_run<BF16>(&plan, g, none, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+       : dtype == OPTIMI_F16
+           ? stable_group_run<F16>(&plan, g, none, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
+           : stable_group_run<F32>(&plan, g, none, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
+  if (rc) return rc;
+  return note_launch(g, stream);
+}
+
+int adan_list(optimi_group* g, int n_tensors, void* const* param, const void* const* grad, void* const* exp_avg,
+              void* const* exp_avg_diff, void* const* exp_avg_sq, void* const* prev_grad, void* const* kahan_comp,
+              const int64_t* numel, const int* dtypes, int dtype, double lr, double beta1_comp, double beta2,
+              double beta2_comp, double beta3_hat, double beta3_comp, double eps, double weight_decay, uint32_t flags,
+              hipStream_t stream) {
+  if (!g) return OPTIMI_ERR_NULL;
+  int rc = resolve_dtypes(n_tensors, &dtypes, &dtype);
+  if (rc) return rc;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const void* const* lists[7] = {(const void* const*)param, grad, (const void* const*)exp_avg,
+                                 (const void* const*)exp_avg_diff, (const void* const*)exp_avg_sq,
+                                 (const void* const*)prev_grad, (const void* const*)kahan_comp};
+  ListPlan plan;
+  rc = plan_list(g, n_tensors, lists, 7, adan_need(kahan, update), bit(6), numel, dtypes, dtype, flags, stream, &plan);
+  if (rc) return rc;
+  if (plan.n_chunks == 0) return 0;
+  const AdanScalars s = adan_scalars(dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay);
+  const AdanScalars s_f32 = adan_scalars(OPTIMI_F32, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay);
+  dispatch<AdanOp, 3>(dtype, kahan, update, adan_wd_mode(weight_decay, flags),
+                      [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream, nullptr, &s_f32); });
+  return finish_list(g, plan, stream);
+}
+
+int sgd_list(optimi_group* g, int n_tensors, void* const* param, const void* const* grad, void* const* exp_avg,
+             void* const* kahan_comp, const int64_t* numel, const int* dtypes, int dtype, double lr, double momentum,
+             double weight_decay, uint32_t flags, hipStream_t stream) {
+  if (!g) return OPTIMI_ERR_NULL;
+  int rc = resolve_dtypes(n_tensors, &dtypes, &dtype);
+  if (rc) return rc;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const int mom = sgd_mom_mode(momentum, flags);
+  if (!update && !mom) return 0;  // nothing to accumulate into
+  const void* const* lists[4] = {(const void* const*)param, grad, (const void* const*)exp_avg, (const void* const*)kahan_comp};
+  ListPlan plan;
+  rc = plan_list(g, n_tensors, lists, 4, sgd_need(kahan, update, mom), bit(3), numel, dtypes, dtype, flags, stream, &plan);
+  if (rc) return rc;
+  if (plan.n_chunks == 0) return 0;
+  const SgdScalars s = sgd_scalars(dtype, lr, momentum, weight_decay);
+  const SgdScalars s_f32 = sgd_scalars(OPTIMI_F32, lr, momentum, weight_decay);
+  sgd_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), mom,
+               [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream, nullptr, &s_f32); });
+  return finish_list(g, plan, stream);
+}
+
+int radam_list(optimi_group* g, int n_tensors, void* const* param, const void* const* grad, void* const* exp_avg,
+               void* const* exp_avg_sq, void* const* kahan_comp, const int64_t* numel, const int* dtypes, int dtype,
+               double lr, double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay, double eps,
+               double rect, uint32_t flags, hipStream_t stream) {
+  if (!g) return OPTIMI_ERR_NULL;
+  int rc = resolve_dtypes(n_tensors, &dtypes, &dtype);
+  if (rc) return rc;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const bool rectify = (flags & OPTIMI_RECTIFY) != 0;
+  const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
+                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
+  ListPlan plan;
+  rc = plan_list(g, n_tensors, lists, 5, adam_need(kahan, update), bit(4), numel, dtypes, dtype, flags, stream, &plan);
+  if (rc) return rc;
+  if (plan.n_chunks == 0) return 0;
+  const double step_lr = rectify ? lr * rect : lr;
+  const AdamScalars s = adam_scalars(dtype, step_lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  const AdamScalars s_f32 = adam_scalars(OPTIMI_F32, step_lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  const int wd = adam_wd_mode(weight_decay, flags);
+  auto launch = [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream, nullptr, &s_f32); };
+  if (rectify || !update) dispatch<AdamOp, 3>(dtype, kahan, update, wd, launch);
+  else dispatch<RAdamEarlyOp, 3>(dtype, kahan, update, wd, launch);
+  return finish_list(g, plan, stream);
+}
+
+int ranger_list(optimi_group* g, int n_tensors, void* const* param, const void* const* grad, void* const* exp_avg,
+                void* const* exp_avg_sq, void* const* la_param, void* const* kahan_comp, const int64_t* numel,
+                const int* dtypes, int dtype, double lr, double beta1_comp, double beta2_hat, double beta2_comp,
+                double weight_decay, double eps, double rect, double alpha, uint32_t flags, hipStream_t stream) {
+  if (!g) return OPTIMI_ERR_NULL;
+  int rc = resolve_dtypes(n_tensors, &dtypes, &dtype);
+  if (rc) return rc;
+  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
+  const bool rectify = (flags & OPTIMI_RECTIFY) != 0, la = (flags & OPTIMI_LOOKAHEAD) != 0;
+  const void* const* lists[6] = {(const void* const*)param, grad, (const void* const*)exp_avg,
+                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp,
+                                 (const void* const*)la_param};
+  ListPlan plan;
+  rc = plan_list(g, n_tensors, lists, 6, ranger_need(kahan, update, la), bit(4), numel, dtypes, dtype, flags, stream, &plan);
+  if (rc) return rc;
+  if (plan.n_chunks == 0) return 0;
+  const double step_lr = rectify ? lr * rect : lr;
+  RangerScalars s, s_f32;
+  s.a = adam_scalars(dtype, step_lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  s.alpha_d = Sd(alpha, dtype);
+  s_f32.a = adam_scalars(OPTIMI_F32, step_lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
+  s_f32.alpha_d = Sd(alpha, OPTIMI_F32);
+  ranger_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), rectify, la,
+                  [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream, nullptr, &s_f32); });
+  return finish_list(g, plan, stream);
+}
+
 }  // namespace
 
 // ------------------------------------------------------------------------------------
@@ -1424,81 +1688,77 @@ int optimi_hip_group_destroy(optimi_group* g) {
 int optimi_hip_adam_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
                           void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
                           const int64_t* numel, int dtype, double lr, double beta1_comp, double beta2_hat,
-                          double beta2_comp, double weight_decay, double eps, uint32_t flags, optimi_stream_t stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
-  const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
-                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
-  ListPlan plan;
-  int rc = plan_list(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, flags, stream, &plan);
-  if (rc) return rc;
-  if (plan.n_chunks == 0) return 0;
-  AdamScalars s = adam_scalars(dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
-  dispatch<AdamOp, 3>(dtype, kahan, update, adam_wd_mode(weight_decay, flags), [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
-  return finish_list(g, plan, stream);
+                          double beta2_comp, double weight_decay, double eps, uint32_t flags, optimi_stream_t stream) {
+  return adam_list(g, n_tensors, param, grad, exp_avg, exp_avg_sq, kahan_comp, numel, nullptr, dtype, lr, beta1_comp,
+                   beta2_hat, beta2_comp, weight_decay, eps, flags, (hipStream_t)stream);
+}
+
+int optimi_hip_adam_multi_mixed(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                                void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                                const int64_t* numel, const int* dtype, double lr, double beta1_comp, double beta2_hat,
+                                double beta2_comp, double weight_decay, double eps, uint32_t flags,
+                                optimi_stream_t stream) {
+  if (!dtype && n_tensors > 0) return OPTIMI_ERR_NULL;
+  return adam_list(g, n_tensors, param, grad, exp_avg, exp_avg_sq, kahan_comp, numel, dtype, OPTIMI_F32, lr, beta1_comp,
+                   beta2_hat, beta2_comp, weight_decay, eps, flags, (hipStream_t)stream);
 }
 
 int optimi_hip_lion_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
                           void* const* exp_avg, void* const* kahan_comp, const int64_t* numel, int dtype, double lr,
                           double beta1_comp, double beta2_comp, double weight_decay, uint32_t flags,
-                          optimi_stream_t stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
-  const void* const* lists[4] = {(const void* const*)param, grad, (const void* const*)exp_avg,
-                                 (const void* const*)kahan_comp};
-  ListPlan plan;
-  int rc = plan_list(g, n_tensors, lists, 4, lion_need(kahan, update), numel, dtype, flags, stream, &plan);
-  if (rc) return rc;
-  if (plan.n_chunks == 0) return 0;
-  LionScalars s = lion_scalars(dtype, lr, beta1_comp, beta2_comp, weight_decay);
-  dispatch<LionOp, 2>(dtype, kahan, update, lion_wd_mode(weight_decay, flags), [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
-  return finish_list(g, plan, stream);
+                          optimi_stream_t stream) {
+  return lion_list(g, n_tensors, param, grad, exp_avg, kahan_comp, numel, nullptr, dtype, lr, beta1_comp, beta2_comp,
+                   weight_decay, flags, (hipStream_t)stream);
+}
+
+int optimi_hip_lion_multi_mixed(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                                void* const* exp_avg, void* const* kahan_comp, const int64_t* numel, const int* dtype,
+                                double lr, double beta1_comp, double beta2_comp, double weight_decay, uint32_t flags,
+                                optimi_stream_t stream) {
+  if (!dtype && n_tensors > 0) return OPTIMI_ERR_NULL;
+  return lion_list(g, n_tensors, param, grad, exp_avg, kahan_comp, numel, dtype, OPTIMI_F32, lr, beta1_comp, beta2_comp,
+                   weight_decay, flags, (hipStream_t)stream);
 }
 
 int optimi_hip_stableadamw_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
                                  void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
                                  const int64_t* numel, int dtype, double lr, double beta1_comp, double beta2_hat,
                                  double beta2_comp, double weight_decay, double eps, double max_lr, uint32_t flags,
-                                 optimi_stream_t stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  if ((flags & OPTIMI_DECOUPLE_LR) && weight_decay != 0 && !(max_lr > 0)) return OPTIMI_ERR_ARG;
-  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
-  const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
-                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
-  ListPlan plan;
-  int rc = plan_list(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, flags, stream, &plan);
-  if (rc) return rc;
-  if (plan.n_chunks == 0) return 0;
-  // the reduction scratch is the group's: a previous launch on another stream may still read it
-  if (plan.few && g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
-  TensorEntry none;
-  std::memset(&none, 0, sizeof(none));
-  rc = dtype == OPTIMI_BF16
-           ? stable_group_run<BF16>(&plan, g, none, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
-       : dtype == OPTIMI_F16
-           ? stable_group_run<F16>(&plan, g, none, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
-           : stable_group_run<F32>(&plan, g, none, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream);
-  if (rc) return rc;
-  return note_launch(g, stream);
+                                 optimi_stream_t stream) {
+  return stableadamw_list(g, n_tensors, param, grad, exp_avg, exp_avg_sq, kahan_comp, numel, nullptr, dtype, lr,
+                          beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, (hipStream_t)stream);
+}
+
+int optimi_hip_stableadamw_multi_mixed(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                                       void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                                       const int64_t* numel, const int* dtype, double lr, double beta1_comp,
+                                       double beta2_hat, double beta2_comp, double weight_decay, double eps,
+                                       double max_lr, uint32_t flags, optimi_stream_t stream) {
+  if (!dtype && n_tensors > 0) return OPTIMI_ERR_NULL;
+  return stableadamw_list(g, n_tensors, param, grad, exp_avg, exp_avg_sq, kahan_comp, numel, dtype, OPTIMI_F32, lr,
+                          beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, (hipStream_t)stream);
 }
 
 int optimi_hip_adan_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
                           void* const* exp_avg, void* const* exp_avg_diff, void* const* exp_avg_sq,
                           void* const* prev_grad, void* const* kahan_comp, const int64_t* numel, int dtype, double lr,
                           double beta1_comp, double beta2, double beta2_comp, double beta3_hat, double beta3_comp,
-                          double eps, double weight_decay, uint32_t flags, optimi_stream_t stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
-  const void* const* lists[7] = {(const void* const*)param, grad, (const void* const*)exp_avg,
-                                 (const void* const*)exp_avg_diff, (const void* const*)exp_avg_sq,
-                                 (const void* const*)prev_grad, (const void* const*)kahan_comp};
-  ListPlan plan;
-  int rc = plan_list(g, n_tensors, lists, 7, adan_need(kahan, update), numel, dtype, flags, stream, &plan);
-  if (rc) return rc;
-  if (plan.n_chunks == 0) return 0;
-  AdanScalars s = adan_scalars(dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay);
-  dispatch<AdanOp, 3>(dtype, kahan, update, adan_wd_mode(weight_decay, flags), [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
-  return finish_list(g, plan, stream);
+                          double eps, double weight_decay, uint32_t flags, optimi_stream_t stream) {
+  return adan_list(g, n_tensors, param, grad, exp_avg, exp_avg_diff, exp_avg_sq, prev_grad, kahan_comp, numel, nullptr,
+                   dtype, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay, flags,
+                   (hipStream_t)stream);
+}
+
+int optimi_hip_adan_multi_mixed(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                                void* const* exp_avg, void* const* exp_avg_diff, void* const* exp_avg_sq,
+                                void* const* prev_grad, void* const* kahan_comp, const int64_t* numel, const int* dtype,
+                                double lr, double beta1_comp, double beta2, double beta2_comp, double beta3_hat,
+                                double beta3_comp, double eps, double weight_decay, uint32_t flags,
+                                optimi_stream_t stream) {
+  if (!dtype && n_tensors > 0) return OPTIMI_ERR_NULL;
+  return adan_list(g, n_tensors, param, grad, exp_avg, exp_avg_diff, exp_avg_sq, prev_grad, kahan_comp, numel, dtype,
+                   OPTIMI_F32, lr, beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay, flags,
+                   (hipStream_t)stream);
 }
 
 int optimi_hip_adam_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* kahan_comp,
@@ -1609,19 +1869,18 @@ int optimi_hip_adan_single(void* param, const void* grad, void* exp_avg, void* e
 
 int optimi_hip_sgd_multi(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
                          void* const* exp_avg, void* const* kahan_comp, const int64_t* numel, int dtype, double lr,
-                         double momentum, double weight_decay, uint32_t flags, optimi_stream_t stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
-  const int mom = sgd_mom_mode(momentum, flags);
-  if (!update && !mom) return g ? 0 : OPTIMI_ERR_NULL;  // nothing to accumulate into
-  const void* const* lists[4] = {(const void* const*)param, grad, (const void* const*)exp_avg, (const void* const*)kahan_comp};
-  ListPlan plan;
-  int rc = plan_list(g, n_tensors, lists, 4, sgd_need(kahan, update, mom), numel, dtype, flags, stream, &plan);
-  if (rc) return rc;
-  if (plan.n_chunks == 0) return 0;
-  SgdScalars s = sgd_scalars(dtype, lr, momentum, weight_decay);
-  sgd_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), mom, [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
-  return finish_list(g, plan, stream);
+                         double momentum, double weight_decay, uint32_t flags, optimi_stream_t stream) {
+  return sgd_list(g, n_tensors, param, grad, exp_avg, kahan_comp, numel, nullptr, dtype, lr, momentum, weight_decay,
+                  flags, (hipStream_t)stream);
+}
+
+int optimi_hip_sgd_multi_mixed(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                               void* const* exp_avg, void* const* kahan_comp, const int64_t* numel, const int* dtype,
+                               double lr, double momentum, double weight_decay, uint32_t flags,
+                               optimi_stream_t stream) {
+  if (!dtype && n_tensors > 0) return OPTIMI_ERR_NULL;
+  return sgd_list(g, n_tensors, param, grad, exp_avg, kahan_comp, numel, dtype, OPTIMI_F32, lr, momentum, weight_decay,
+                  flags, (hipStream_t)stream);
 }
 
 int optimi_hip_sgd_single(void* param, const void* grad, void* exp_avg, void* kahan_comp, int64_t numel, int dtype,
@@ -1644,21 +1903,19 @@ int optimi_hip_radam_multi(optimi_group* g, int n_tensors, void* const* param, c
                            void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
                            const int64_t* numel, int dtype, double lr, double beta1_comp, double beta2_hat,
                            double beta2_comp, double weight_decay, double eps, double rect, uint32_t flags,
-                           optimi_stream_t stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
-  const bool rectify = (flags & OPTIMI_RECTIFY) != 0;
-  const void* const* lists[5] = {(const void* const*)param, grad, (const void* const*)exp_avg,
-                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp};
-  ListPlan plan;
-  int rc = plan_list(g, n_tensors, lists, 5, adam_need(kahan, update), numel, dtype, flags, stream, &plan);
-  if (rc) return rc;
-  if (plan.n_chunks == 0) return 0;
-  AdamScalars s = adam_scalars(dtype, rectify ? lr * rect : lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
-  const int wd = adam_wd_mode(weight_decay, flags);
-  if (rectify || !update) dispatch<AdamOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
-  else dispatch<RAdamEarlyOp, 3>(dtype, kahan, update, wd, [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
-  return finish_list(g, plan, stream);
+                           optimi_stream_t stream) {
+  return radam_list(g, n_tensors, param, grad, exp_avg, exp_avg_sq, kahan_comp, numel, nullptr, dtype, lr, beta1_comp,
+                    beta2_hat, beta2_comp, weight_decay, eps, rect, flags, (hipStream_t)stream);
+}
+
+int optimi_hip_radam_multi_mixed(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                                 void* const* exp_avg, void* const* exp_avg_sq, void* const* kahan_comp,
+                                 const int64_t* numel, const int* dtype, double lr, double beta1_comp, double beta2_hat,
+                                 double beta2_comp, double weight_decay, double eps, double rect, uint32_t flags,
+                                 optimi_stream_t stream) {
+  if (!dtype && n_tensors > 0) return OPTIMI_ERR_NULL;
+  return radam_list(g, n_tensors, param, grad, exp_avg, exp_avg_sq, kahan_comp, numel, dtype, OPTIMI_F32, lr, beta1_comp,
+                    beta2_hat, beta2_comp, weight_decay, eps, rect, flags, (hipStream_t)stream);
 }
 
 int optimi_hip_radam_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* kahan_comp,
@@ -1685,23 +1942,19 @@ int optimi_hip_ranger_multi(optimi_group* g, int n_tensors, void* const* param, 
                             void* const* exp_avg, void* const* exp_avg_sq, void* const* la_param,
                             void* const* kahan_comp, const int64_t* numel, int dtype, double lr, double beta1_comp,
                             double beta2_hat, double beta2_comp, double weight_decay, double eps, double rect,
-                            double alpha, uint32_t flags, optimi_stream_t stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  const bool update = (flags & OPTIMI_UPDATE) != 0, kahan = kahan_on(dtype, flags);
-  const bool rectify = (flags & OPTIMI_RECTIFY) != 0, la = (flags & OPTIMI_LOOKAHEAD) != 0;
-  const void* const* lists[6] = {(const void* const*)param, grad, (const void* const*)exp_avg,
-                                 (const void* const*)exp_avg_sq, (const void* const*)kahan_comp,
-                                 (const void* const*)la_param};
-  ListPlan plan;
-  int rc = plan_list(g, n_tensors, lists, 6, ranger_need(kahan, update, la), numel, dtype, flags, stream, &plan);
-  if (rc) return rc;
-  if (plan.n_chunks == 0) return 0;
-  RangerScalars s;
-  s.a = adam_scalars(dtype, rectify ? lr * rect : lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
-  s.alpha_d = Sd(alpha, dtype);
-  ranger_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), rectify, la,
-                  [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream); });
-  return finish_list(g, plan, stream);
+                            double alpha, uint32_t flags, optimi_stream_t stream) {
+  return ranger_list(g, n_tensors, param, grad, exp_avg, exp_avg_sq, la_param, kahan_comp, numel, nullptr, dtype, lr,
+                     beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, rect, alpha, flags, (hipStream_t)stream);
+}
+
+int optimi_hip_ranger_multi_mixed(optimi_group* g, int n_tensors, void* const* param, const void* const* grad,
+                                  void* const* exp_avg, void* const* exp_avg_sq, void* const* la_param,
+                                  void* const* kahan_comp, const int64_t* numel, const int* dtype, double lr,
+                                  double beta1_comp, double beta2_hat, double beta2_comp, double weight_decay,
+                                  double eps, double rect, double alpha, uint32_t flags, optimi_stream_t stream) {
+  if (!dtype && n_tensors > 0) return OPTIMI_ERR_NULL;
+  return ranger_list(g, n_tensors, param, grad, exp_avg, exp_avg_sq, la_param, kahan_comp, numel, dtype, OPTIMI_F32, lr,
+                     beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, rect, alpha, flags, (hipStream_t)stream);
 }
 
 int optimi_hip_ranger_single(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, void* la_param,
@@ -1733,9 +1986,12 @@ int optimi_hip_copy_probe(void* dst, const void* src, int64_t bytes, optimi_stre
   if (n_vec == 0) return 0;
   const int64_t blocks = (n_vec + 255) / 256;
   if (blocks > 0x7fffffff) return OPTIMI_ERR_SIZE;
+  ++kernel_launches;
   copy_probe_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream_>>>((u32x4*)dst, (const u32x4*)src, n_vec);
   HIP_TRY(hipGetLastError());
   return 0;
 }
+
+int64_t optimi_hip_launch_count(void) { return kernel_launches.load(); }
 
 }  // extern "C"

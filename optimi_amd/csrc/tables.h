@@ -3,8 +3,9 @@
 // a CPU build (with sanitizers) can exercise exactly the code the library runs; the functions
 // the kernels share are marked OPTIMI_HD.
 //
-// A list of tensors is cut into chunks of kChunkBytes per array; chunks are numbered through
-// the whole list, tensor after tensor, and kSub workgroups share a chunk.  A workgroup learns
+// A list of tensors is cut into chunks of kChunkBytes per array (so a chunk of an fp32 tensor
+// holds half the elements of a chunk of a 16-bit one); chunks are numbered through the whole
+// list, tensor after tensor, and kSub workgroups share a chunk.  A workgroup learns
 // which tensor its chunk belongs to either from a chunk map in device memory (large lists) or,
 // for lists of at most kFew tensors, by searching a table that travels as a kernel argument.
 // This takes the place of the per-tensor Python launch loops of the reference
@@ -40,6 +41,7 @@ struct TensorEntry {
 };
 constexpr uint32_t kEntryVec = 1;     // all buffers 16-byte aligned: the vector path applies
 constexpr uint32_t kEntryCached = 2;  // read full tiles with ordinary cached loads instead of streaming ones
+constexpr uint32_t kEntryF32 = 4;     // the tensor is fp32 (a list may mix fp32 tensors with tensors of one 16-bit dtype)
 static_assert(sizeof(TensorEntry) == 80, "TensorEntry layout");
 
 struct FewTable {
@@ -56,30 +58,39 @@ inline int elem_bytes(int dtype) { return dtype == OPTIMI_F32 ? 4 : 2; }
 inline int64_t chunk_elems(int dtype) { return kChunkBytes / elem_bytes(dtype); }
 inline int64_t chunks_of(int64_t numel, int64_t chunk) { return (numel + chunk - 1) / chunk; }
 
+inline int64_t entry_chunk_elems(const TensorEntry& e) { return kChunkBytes / ((e.flags & kEntryF32) ? 4 : 2); }
+
 // Validates a list and writes one entry per tensor.  `lists[a]` may be nullptr for an array the
-// launch does not touch (`need` has its bit clear).  `max_chunks` bounds the launch (the grid
-// is chunks x workgroups per chunk and must fit 31 bits).  Returns an optimi_status.
+// launch does not touch (`need` has its bit clear).  `dtypes`, when not null, gives every
+// tensor's own dtype (a mixed list); otherwise all tensors have `dtype`.  Arrays in
+// `low_precision_only` (the Kahan buffer) exist for 16-bit tensors only: an fp32 tensor's
+// pointer there is ignored.  `max_chunks` bounds the launch (the grid is chunks x workgroups
+// per chunk and must fit 31 bits).  Returns an optimi_status.
 inline int build_entries(int n_tensors, const void* const* const* lists, int n_arrays, uint32_t need, const int64_t* numel,
-                         int dtype, int64_t max_chunks, TensorEntry* out, int64_t* n_chunks_out) {
+                         const int* dtypes, int dtype, uint32_t low_precision_only, int64_t max_chunks, TensorEntry* out,
+                         int64_t* n_chunks_out) {
   if (n_tensors < 0) return OPTIMI_ERR_SIZE;
-  if (!valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
+  if (!dtypes && !valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
   if (n_arrays < 0 || n_arrays > kMaxArrays) return OPTIMI_ERR_SIZE;
   if (n_tensors > 0 && (!numel || !out)) return OPTIMI_ERR_NULL;
   for (int a = 0; a < n_arrays; ++a)
     if ((need & bit(a)) && n_tensors > 0 && (!lists || !lists[a])) return OPTIMI_ERR_NULL;
-  const int64_t chunk = chunk_elems(dtype);
-  const uintptr_t eb = (uintptr_t)elem_bytes(dtype);
   int64_t n_chunks = 0;
   for (int t = 0; t < n_tensors; ++t) {
+    const int dt = dtypes ? dtypes[t] : dtype;
+    if (!valid_dtype(dt)) return OPTIMI_ERR_DTYPE;
+    const int64_t chunk = chunk_elems(dt);
+    const uintptr_t eb = (uintptr_t)elem_bytes(dt);
     TensorEntry& e = out[t];
     std::memset(&e, 0, sizeof(e));
     if (numel[t] < 0) return OPTIMI_ERR_SIZE;
     if (numel[t] > max_chunks * chunk) return OPTIMI_ERR_SIZE;  // also keeps the sums below from overflowing
     e.numel = numel[t];
     e.first_chunk = n_chunks;
-    e.flags = kEntryVec;
+    e.flags = kEntryVec | (dt == OPTIMI_F32 ? kEntryF32 : 0u);
     for (int a = 0; a < n_arrays; ++a) {
       if (!(need & bit(a))) continue;
+      if (dt == OPTIMI_F32 && (low_precision_only & bit(a))) continue;
       const void* p = lists[a][t];
       if (!p && numel[t] > 0) return OPTIMI_ERR_NULL;
       const uintptr_t u = (uintptr_t)p;
@@ -95,9 +106,9 @@ inline int build_entries(int n_tensors, const void* const* const* lists, int n_a
 }
 
 // chunk -> tensor for every chunk of the launch; `map` has room for the launch's chunk count.
-inline void build_chunk_map(const TensorEntry* entries, int n_tensors, int64_t chunk, int32_t* map) {
+inline void build_chunk_map(const TensorEntry* entries, int n_tensors, int32_t* map) {
   for (int t = 0; t < n_tensors; ++t) {
-    const int64_t c0 = entries[t].first_chunk, c1 = c0 + chunks_of(entries[t].numel, chunk);
+    const int64_t c0 = entries[t].first_chunk, c1 = c0 + chunks_of(entries[t].numel, entry_chunk_elems(entries[t]));
     for (int64_t c = c0; c < c1; ++c) map[c] = t;
   }
 }

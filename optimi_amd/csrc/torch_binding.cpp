@@ -93,42 +93,54 @@ PtrList gather(const TensorList& params, const TensorList& list, const char* nam
   return out;
 }
 
-// Kahan buffers: taken only when the Kahan branch runs; placeholders and None are ignored.
-PtrList gather_kahan(const TensorList& params, const OptTensorList& list, bool needed) {
+struct Prepared {
+  std::vector<int> dtypes;  // every tensor's dtype: fp32 and at most one 16-bit dtype
+  bool kahan = false;       // the Kahan branch runs for the 16-bit tensors
+  std::vector<int64_t> numel;
+  PtrList params;
+};
+
+// One launch covers one device; its tensors are fp32 or of one 16-bit dtype, in any mixture.
+Prepared prepare(const TensorList& params, uint32_t flags) {
+  Prepared pr;
+  if (params.empty()) return pr;
+  pr.numel.reserve(params.size());
+  pr.dtypes.reserve(params.size());
+  pr.params.v.reserve(params.size());
+  int low = OPTIMI_F32;
+  for (const at::Tensor& p : params) {
+    check_param(p);
+    TORCH_CHECK(p.device() == params[0].device(), "optimi_amd: one launch covers one device");
+    const int dtype = dtype_code(p);
+    if (dtype != OPTIMI_F32) {
+      TORCH_CHECK(low == OPTIMI_F32 || low == dtype, "optimi_amd: one launch covers float32 and one 16-bit dtype, not bfloat16 and float16 together");
+      low = dtype;
+    }
+    pr.dtypes.push_back(dtype);
+    pr.numel.push_back(p.numel());
+    pr.params.v.push_back(p.data_ptr());
+  }
+  pr.kahan = low != OPTIMI_F32 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
+  return pr;
+}
+
+// Kahan buffers: taken only when the Kahan branch runs, and only for the 16-bit tensors;
+// placeholders and None are ignored.
+PtrList gather_kahan(const TensorList& params, const OptTensorList& list, const Prepared& pr) {
   PtrList out;
-  if (!needed) return out;
+  if (!pr.kahan) return out;
   TORCH_CHECK(list.size() == params.size(), "optimi_amd: kahan_comps has ", list.size(), " tensors, params has ", params.size());
   out.v.reserve(list.size());
   for (size_t i = 0; i < list.size(); ++i) {
+    if (pr.dtypes[i] == OPTIMI_F32) {
+      out.v.push_back(nullptr);
+      continue;
+    }
     TORCH_CHECK(list[i].has_value(), "optimi_amd: kahan_sum is on but a Kahan buffer is missing");
     check_like(params[i], *list[i], "kahan_comp");
     out.v.push_back(list[i]->data_ptr());
   }
   return out;
-}
-
-struct Prepared {
-  int dtype = OPTIMI_F32;
-  bool kahan = false;
-  std::vector<int64_t> numel;
-  PtrList params;
-};
-
-Prepared prepare(const TensorList& params, uint32_t flags) {
-  Prepared pr;
-  if (params.empty()) return pr;
-  pr.dtype = dtype_code(params[0]);
-  pr.kahan = pr.dtype != OPTIMI_F32 && (flags & OPTIMI_KAHAN) && (flags & OPTIMI_UPDATE);
-  pr.numel.reserve(params.size());
-  pr.params.v.reserve(params.size());
-  for (const at::Tensor& p : params) {
-    check_param(p);
-    TORCH_CHECK(p.device() == params[0].device(), "optimi_amd: one launch covers one device");
-    TORCH_CHECK(p.scalar_type() == params[0].scalar_type(), "optimi_amd: one launch covers one dtype");
-    pr.numel.push_back(p.numel());
-    pr.params.v.push_back(p.data_ptr());
-  }
-  return pr;
 }
 
 void adam_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
@@ -137,12 +149,12 @@ void adam_multi(Group& group, const TensorList& params, const TensorList& grads,
   if (params.empty()) return;
   Prepared pr = prepare(params, flags);
   PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
-  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  PtrList k = gather_kahan(params, kahan_comps, pr);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
-  check_status(optimi_hip_adam_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
-                                     pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp, beta2_hat,
+  check_status(optimi_hip_adam_multi_mixed(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
+                                     pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtypes.data(), lr, beta1_comp, beta2_hat,
                                      beta2_comp, weight_decay, eps, flags, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
-               "optimi_hip_adam_multi");
+               "optimi_hip_adam_multi_mixed");
 }
 
 void lion_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
@@ -151,12 +163,12 @@ void lion_multi(Group& group, const TensorList& params, const TensorList& grads,
   if (params.empty()) return;
   Prepared pr = prepare(params, flags);
   PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg");
-  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  PtrList k = gather_kahan(params, kahan_comps, pr);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
-  check_status(optimi_hip_lion_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(),
-                                     pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp, beta2_comp,
+  check_status(optimi_hip_lion_multi_mixed(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(),
+                                     pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtypes.data(), lr, beta1_comp, beta2_comp,
                                      weight_decay, flags, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
-               "optimi_hip_lion_multi");
+               "optimi_hip_lion_multi_mixed");
 }
 
 void stableadamw_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
@@ -166,13 +178,13 @@ void stableadamw_multi(Group& group, const TensorList& params, const TensorList&
   if (params.empty()) return;
   Prepared pr = prepare(params, flags);
   PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
-  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  PtrList k = gather_kahan(params, kahan_comps, pr);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
-  check_status(optimi_hip_stableadamw_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
-                                            pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp,
+  check_status(optimi_hip_stableadamw_multi_mixed(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
+                                            pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtypes.data(), lr, beta1_comp,
                                             beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags,
                                             c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
-               "optimi_hip_stableadamw_multi");
+               "optimi_hip_stableadamw_multi_mixed");
 }
 
 void adan_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
@@ -184,13 +196,13 @@ void adan_multi(Group& group, const TensorList& params, const TensorList& grads,
   PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg");
   PtrList df = gather(params, exp_avg_diffs, "exp_avg_diff"), n = gather(params, exp_avg_sqs, "exp_avg_sq");
   PtrList pg = gather(params, prev_grads, "prev_grad");
-  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  PtrList k = gather_kahan(params, kahan_comps, pr);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
-  check_status(optimi_hip_adan_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), df.data(),
-                                     n.data(), pg.data(), pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr,
+  check_status(optimi_hip_adan_multi_mixed(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), df.data(),
+                                     n.data(), pg.data(), pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtypes.data(), lr,
                                      beta1_comp, beta2, beta2_comp, beta3_hat, beta3_comp, eps, weight_decay, flags,
                                      c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
-               "optimi_hip_adan_multi");
+               "optimi_hip_adan_multi_mixed");
 }
 
 // Momentum buffers: absent (None or a one-element placeholder) when SGD runs without momentum.
@@ -213,13 +225,13 @@ void sgd_multi(Group& group, const TensorList& params, const TensorList& grads, 
   Prepared pr = prepare(params, flags);
   PtrList g = gather(params, grads, "grad");
   PtrList m = gather_optional(params, exp_avgs, momentum != 0, "exp_avg");
-  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  PtrList k = gather_kahan(params, kahan_comps, pr);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
-  check_status(optimi_hip_sgd_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(),
+  check_status(optimi_hip_sgd_multi_mixed(group.get(), (int)params.size(), pr.params.data(), g.cdata(),
                                     momentum != 0 ? m.data() : nullptr, pr.kahan ? k.data() : nullptr, pr.numel.data(),
-                                    pr.dtype, lr, momentum, weight_decay, flags,
+                                    pr.dtypes.data(), lr, momentum, weight_decay, flags,
                                     c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
-               "optimi_hip_sgd_multi");
+               "optimi_hip_sgd_multi_mixed");
 }
 
 void radam_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
@@ -228,13 +240,13 @@ void radam_multi(Group& group, const TensorList& params, const TensorList& grads
   if (params.empty()) return;
   Prepared pr = prepare(params, flags);
   PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
-  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  PtrList k = gather_kahan(params, kahan_comps, pr);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
-  check_status(optimi_hip_radam_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
-                                      pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp, beta2_hat,
+  check_status(optimi_hip_radam_multi_mixed(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
+                                      pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtypes.data(), lr, beta1_comp, beta2_hat,
                                       beta2_comp, weight_decay, eps, rect, flags,
                                       c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
-               "optimi_hip_radam_multi");
+               "optimi_hip_radam_multi_mixed");
 }
 
 void ranger_multi(Group& group, const TensorList& params, const TensorList& grads, const TensorList& exp_avgs,
@@ -245,13 +257,13 @@ void ranger_multi(Group& group, const TensorList& params, const TensorList& grad
   Prepared pr = prepare(params, flags);
   PtrList g = gather(params, grads, "grad"), m = gather(params, exp_avgs, "exp_avg"), v = gather(params, exp_avg_sqs, "exp_avg_sq");
   PtrList la = gather(params, la_params, "la_param");
-  PtrList k = gather_kahan(params, kahan_comps, pr.kahan);
+  PtrList k = gather_kahan(params, kahan_comps, pr);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(params[0].device());
-  check_status(optimi_hip_ranger_multi(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
-                                       la.data(), pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtype, lr, beta1_comp,
+  check_status(optimi_hip_ranger_multi_mixed(group.get(), (int)params.size(), pr.params.data(), g.cdata(), m.data(), v.data(),
+                                       la.data(), pr.kahan ? k.data() : nullptr, pr.numel.data(), pr.dtypes.data(), lr, beta1_comp,
                                        beta2_hat, beta2_comp, weight_decay, eps, rect, alpha, flags,
                                        c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
-               "optimi_hip_ranger_multi");
+               "optimi_hip_ranger_multi_mixed");
 }
 
 // ---- per-tensor entry points (gradient release) --------------------------------------
@@ -456,48 +468,52 @@ void launch_now(const StepCall& c, Group* stable_group) {
 }
 
 // One whole-list launch of `kind`: ptr[a][i] is tensor i of array a, in the ABI's order for
-// that kind; an array whose first pointer is NULL is passed as absent (Kahan buffers when the
-// Kahan branch is off, SGD's momentum buffer without momentum).
-void launch_list(Kind kind, optimi_group* g, int n, const std::vector<void*>* ptr, const int64_t* numel, int dtype,
+// that kind, dtypes[i] its dtype; an array without any pointer is passed as absent (Kahan
+// buffers when the Kahan branch is off, SGD's momentum buffer without momentum).
+void launch_list(Kind kind, optimi_group* g, int n, const std::vector<void*>* ptr, const int64_t* numel, const int* dtypes,
                  const double* s, uint32_t flags, hipStream_t stream) {
   auto arr = [&](int a) { return (void* const*)ptr[a].data(); };
   auto carr = [&](int a) { return (const void* const*)ptr[a].data(); };
-  auto opt = [&](int a) { return (n > 0 && ptr[a][0]) ? (void* const*)ptr[a].data() : nullptr; };
+  auto opt = [&](int a) -> void* const* {
+    for (void* q : ptr[a])
+      if (q) return (void* const*)ptr[a].data();
+    return nullptr;
+  };
   int rc = 0;
   const char* what = "";
   switch (kind) {
     case ADAM:
-      rc = optimi_hip_adam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype,
+      rc = optimi_hip_adam_multi_mixed(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtypes,
           s[0], s[1], s[2], s[3], s[4], s[5], flags, stream);
-      what = "optimi_hip_adam_multi";
+      what = "optimi_hip_adam_multi_mixed";
       break;
     case LION:
-      rc = optimi_hip_lion_multi(g, n, arr(0), carr(1), arr(2), opt(3), numel, dtype, s[0], s[1], s[2], s[3], flags, stream);
-      what = "optimi_hip_lion_multi";
+      rc = optimi_hip_lion_multi_mixed(g, n, arr(0), carr(1), arr(2), opt(3), numel, dtypes, s[0], s[1], s[2], s[3], flags, stream);
+      what = "optimi_hip_lion_multi_mixed";
       break;
     case STABLEADAMW:
-      rc = optimi_hip_stableadamw_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype,
+      rc = optimi_hip_stableadamw_multi_mixed(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtypes,
           s[0], s[1], s[2], s[3], s[4], s[5], s[6], flags, stream);
-      what = "optimi_hip_stableadamw_multi";
+      what = "optimi_hip_stableadamw_multi_mixed";
       break;
     case ADAN:
-      rc = optimi_hip_adan_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), arr(5), opt(6), numel, dtype,
+      rc = optimi_hip_adan_multi_mixed(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), arr(5), opt(6), numel, dtypes,
           s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], flags, stream);
-      what = "optimi_hip_adan_multi";
+      what = "optimi_hip_adan_multi_mixed";
       break;
     case SGD:
-      rc = optimi_hip_sgd_multi(g, n, arr(0), carr(1), opt(2), opt(3), numel, dtype, s[0], s[1], s[2], flags, stream);
-      what = "optimi_hip_sgd_multi";
+      rc = optimi_hip_sgd_multi_mixed(g, n, arr(0), carr(1), opt(2), opt(3), numel, dtypes, s[0], s[1], s[2], flags, stream);
+      what = "optimi_hip_sgd_multi_mixed";
       break;
     case RADAM:
-      rc = optimi_hip_radam_multi(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtype,
+      rc = optimi_hip_radam_multi_mixed(g, n, arr(0), carr(1), arr(2), arr(3), opt(4), numel, dtypes,
           s[0], s[1], s[2], s[3], s[4], s[5], s[6], flags, stream);
-      what = "optimi_hip_radam_multi";
+      what = "optimi_hip_radam_multi_mixed";
       break;
     case RANGER:
-      rc = optimi_hip_ranger_multi(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), opt(5), numel, dtype,
+      rc = optimi_hip_ranger_multi_mixed(g, n, arr(0), carr(1), arr(2), arr(3), arr(4), opt(5), numel, dtypes,
           s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7], flags, stream);
-      what = "optimi_hip_ranger_multi";
+      what = "optimi_hip_ranger_multi_mixed";
       break;
   }
   check_status(rc, what);
@@ -519,8 +535,9 @@ void check_hip(hipError_t err, const char* what) {
 }
 
 // Parks the steps of small tensors and launches them together, as one list per run of steps
-// that share everything but their tensors (optimizer, dtype, device, stream, flags and every
-// scalar - which includes the step count through the debiased betas).  A tensor of a few
+// that share everything but their tensors (optimizer, device, stream, flags and every scalar -
+// which includes the step count through the debiased betas; fp32 tensors and tensors of one
+// 16-bit dtype share a list, so a bf16 model with fp32 norms does not break the run at every norm).  A tensor of a few
 // thousand elements costs far more to launch than to update, so a model with thousands of
 // them is bound by launches; one list launch replaces up to `max_tensors` of them.  The queue
 // keeps each parked gradient alive until its launch; `max_total` bounds how many bytes of
@@ -576,7 +593,11 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
     std::lock_guard<std::recursive_mutex> lock(mutex_);
     const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(c.param().device().index()).stream();
     if (!batch_.empty() && (!same_run(c, stream) || seen_.count(c.param().data_ptr()))) flush();
-    if (batch_.empty()) stream_ = stream;
+    if (batch_.empty()) {
+      stream_ = stream;
+      low_dtype_ = at::kFloat;
+    }
+    if (c.param().scalar_type() != at::kFloat) low_dtype_ = c.param().scalar_type();
     total_ += c.param().numel() * (int64_t)c.param().element_size();
     seen_.insert(c.param().data_ptr());
     batch_.push_back(std::move(c));
@@ -606,12 +627,13 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
     }
     const StepCall& c0 = batch[0];
     const int n = (int)batch.size(), nt = kTensorsOf[c0.kind];
-    const int dtype = dtype_code(c0.param());
     std::vector<void*> ptr[kMaxTensors];
     std::vector<int64_t> numel((size_t)n);
+    std::vector<int> dtypes((size_t)n);
     for (int a = 0; a < nt; ++a) ptr[a].resize((size_t)n, nullptr);
     for (int i = 0; i < n; ++i) {
       numel[(size_t)i] = batch[(size_t)i].param().numel();
+      dtypes[(size_t)i] = dtype_code(batch[(size_t)i].param());
       for (int a = 0; a < nt; ++a)
         if (batch[(size_t)i].t[a].has_value()) ptr[a][(size_t)i] = batch[(size_t)i].t[a]->data_ptr();
     }
@@ -629,7 +651,7 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
     }
     // OPTIMI_COLD: these tensors are a slice of a model whose backward pass has just streamed
     // through the caches; a short list must not be taken for a small resident model
-    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtype, c0.s, c0.flags | OPTIMI_COLD, launch);
+    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtypes.data(), c0.s, c0.flags | OPTIMI_COLD, launch);
     ++launches_;
     launched_steps_ += n;
     if (launch != current) {
@@ -647,9 +669,12 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
   bool same_run(const StepCall& c, hipStream_t stream) const {
     const StepCall& c0 = batch_[0];
     if (c.kind != c0.kind || c.flags != c0.flags || stream != stream_) return false;
-    if (c.param().scalar_type() != c0.param().scalar_type() || c.param().device() != c0.param().device()) return false;
+    if (c.param().device() != c0.param().device()) return false;
+    const at::ScalarType dtype = c.param().scalar_type();
+    if (dtype != at::kFloat && low_dtype_ != at::kFloat && dtype != low_dtype_) return false;  // bf16 and fp16 do not share a list
     if (std::memcmp(c.s, c0.s, sizeof(c.s)) != 0) return false;
-    for (int a = 0; a < kTensorsOf[c.kind]; ++a)
+    // the same arrays present, except the Kahan buffer (the last one), which fp32 tensors never have
+    for (int a = 0; a < kTensorsOf[c.kind] - 1; ++a)
       if (c.t[a].has_value() != c0.t[a].has_value()) return false;
     return true;
   }
@@ -663,6 +688,7 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
   std::unordered_set<void*> seen_;
   int64_t total_ = 0;
   hipStream_t stream_ = nullptr;
+  at::ScalarType low_dtype_ = at::kFloat;  // the 16-bit dtype among the parked tensors, float while there is none
   std::atomic<int64_t> launches_{0}, launched_steps_{0};
 };
 
@@ -875,7 +901,7 @@ class ReleaseHookCore {
 
   // One whole-group step (optimi/adam.py:158-182 and the functional form behind it) without the
   // per-parameter Python walk: collects the parameters of `group` that have a gradient, advances
-  // the group's step counter, forms the scalars and launches one list per (device, dtype).
+  // the group's step counter, forms the scalars and launches one list per device.
   // Returns false, having done nothing, when the group has not been set up yet (the first step
   // goes through Python, which resolves the backend) - the caller then takes the Python path.
   bool step_group(const py::dict& group) {
@@ -920,29 +946,45 @@ class ReleaseHookCore {
     if (items.empty()) return true;
     const Hyper h = read_hyper(grp, t, true);
 
-    // pass 2: one launch per (device, dtype), in order of first appearance
+    // pass 2: one launch per device, in order of first appearance.  fp32 parameters and the
+    // parameters of one 16-bit dtype go together; a group that holds bf16 and fp16 gets a launch for each.
     const int nt = kTensorsOf[kind_];
     std::vector<char> done(items.size(), 0);
     for (size_t first = 0; first < items.size(); ++first) {
       if (done[first]) continue;
       const at::Tensor& p0 = items[first].p;
+      at::ScalarType low = at::kFloat;
       std::vector<void*> ptr[kMaxTensors];
       std::vector<int64_t> numel;
+      std::vector<int> dtypes;
       for (size_t i = first; i < items.size(); ++i) {
         const at::Tensor& p = items[i].p;
-        if (done[i] || p.scalar_type() != p0.scalar_type() || p.device() != p0.device()) continue;
+        if (done[i] || p.device() != p0.device()) continue;
+        if (p.scalar_type() != at::kFloat) {
+          if (low != at::kFloat && p.scalar_type() != low) continue;
+          low = p.scalar_type();
+        }
         done[i] = 1;
         const StepCall c = pack(*items[i].e, h, p, items[i].g, momentum);
         for (int a = 0; a < nt; ++a) ptr[a].push_back(c.t[a].has_value() ? c.t[a]->data_ptr() : nullptr);
+        if (p.scalar_type() == at::kFloat) ptr[nt - 1].back() = nullptr;  // no Kahan buffer for fp32
         numel.push_back(p.numel());
+        dtypes.push_back(dtype_code(p));
       }
-      // an absent array must be absent for every tensor of the launch
-      for (int a = 2; a < nt; ++a)
-        for (void* q : ptr[a]) TORCH_CHECK((q == nullptr) == (ptr[a][0] == nullptr), "optimi_amd: a state buffer is missing for some parameters of a group");
+      // an absent array must be absent for every tensor of the launch (the Kahan buffer: for every 16-bit one)
+      for (int a = 2; a < nt; ++a) {
+        int present = -1;
+        for (size_t i = 0; i < ptr[a].size(); ++i) {
+          if (a == nt - 1 && dtypes[i] == OPTIMI_F32) continue;
+          const int here = ptr[a][i] != nullptr;
+          TORCH_CHECK(present < 0 || present == here, "optimi_amd: a state buffer is missing for some parameters of a group");
+          present = here;
+        }
+      }
       c10::hip::HIPGuardMasqueradingAsCUDA guard(p0.device());
-      std::unique_ptr<Group>& slot = workspaces_[{(int)p0.device().index(), (int)p0.scalar_type()}];
+      std::unique_ptr<Group>& slot = workspaces_[{(int)p0.device().index(), (int)low}];
       if (!slot) slot = std::make_unique<Group>();
-      launch_list(kind_, slot->get(), (int)numel.size(), ptr, numel.data(), dtype_code(p0), h.s, h.flags,
+      launch_list(kind_, slot->get(), (int)numel.size(), ptr, numel.data(), dtypes.data(), h.s, h.flags,
                   c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(p0.device().index()).stream());
     }
     return true;
@@ -1138,7 +1180,7 @@ class ReleaseHookCore {
   struct PairHash {
     size_t operator()(const std::pair<int, int>& k) const { return std::hash<int64_t>()(((int64_t)k.first << 32) ^ (int64_t)k.second); }
   };
-  std::unordered_map<std::pair<int, int>, std::unique_ptr<Group>, PairHash> workspaces_;  // (device, dtype) -> tables
+  std::unordered_map<std::pair<int, int>, std::unique_ptr<Group>, PairHash> workspaces_;  // (device, 16-bit dtype of the list or float) -> tables
 };
 
 // What is registered on the parameters: a handle that does not own the hook, so that

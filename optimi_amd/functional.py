@@ -59,11 +59,19 @@ def _as_lists(*cols):
 
 
 def _buckets(params: list[Tensor]):
-    """Indices of ``params`` grouped by (device, dtype): one launch each."""
+    """Indices of ``params`` grouped into launches: one per device, float32 tensors together with the
+    tensors of one 16-bit dtype.  Keys are (device, that 16-bit dtype or float32); a device that
+    holds bfloat16 and float16 parameters gets a launch for each, the float32 ones riding with
+    whichever 16-bit dtype comes first."""
+    low = {}
+    for p in params:
+        backend.check_supported(p)
+        if p.dtype != torch.float32:
+            low.setdefault(p.device, p.dtype)
     out = defaultdict(list)
     for i, p in enumerate(params):
-        backend.check_supported(p)
-        out[(p.device, p.dtype)].append(i)
+        dtype = low.get(p.device, torch.float32) if p.dtype == torch.float32 else p.dtype
+        out[(p.device, dtype)].append(i)
     return out
 
 

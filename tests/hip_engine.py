@@ -8,6 +8,8 @@ torch only provides device memory and the stream here: every launch goes through
 
 from __future__ import annotations
 
+import ctypes as C
+
 import torch
 
 from optimi_amd import cabi
@@ -22,12 +24,15 @@ def _addr(t):
 
 
 class HipRun(ForLoopRun):
-    """``multi=True``: whole-list entry points (one launch); False: per-tensor entry points."""
+    """``multi=True``: whole-list entry points (one launch); False: per-tensor entry points.
+    A list whose tensors differ in dtype goes through the ``_multi_mixed`` entry points;
+    ``mixed=True`` sends a list of one dtype through them as well."""
 
-    def __init__(self, name, params, *, multi=True, cold=False, **kw):
+    def __init__(self, name, params, *, multi=True, cold=False, mixed=False, **kw):
         super().__init__(name, params, **kw)
         self.multi = multi
         self.cold = cold  # pass OPTIMI_COLD to the whole-list entry points
+        self.mixed = mixed
         self.group = cabi.Group()
         self.entry = "adam" if name == "adamw" else name
 
@@ -70,7 +75,11 @@ class HipRun(ForLoopRun):
             cols = [cabi.ptr_array(_addr(p) for p in ps), cabi.ptr_array(_addr(g) for g in grads)]
             cols += [cabi.ptr_array(_addr(s[k]) for s in sts) for k in STATE_ORDER[self.name]]
             cols.append(cabi.ptr_array(_addr(s["kahan_comp"]) for s in sts))
-            fn = getattr(L, f"optimi_hip_{self.entry}_multi")
+            if self.mixed or len({p.dtype for p in ps}) > 1:
+                fn = getattr(L, f"optimi_hip_{self.entry}_multi_mixed")
+                dt = (C.c_int * len(ps))(*[DT[p.dtype] for p in ps])
+            else:
+                fn = getattr(L, f"optimi_hip_{self.entry}_multi")
             rc = fn(self.group.handle, len(ps), *cols, cabi.i64_array(p.numel() for p in ps), dt, *scalars, self._stream())
             cabi.check(rc, fn.__name__)
         else:
@@ -78,7 +87,7 @@ class HipRun(ForLoopRun):
             lead = (self.group.handle,) if self.entry == "stableadamw" else ()
             for p, g, s in zip(ps, grads, sts):
                 bufs = [_addr(s[k]) for k in STATE_ORDER[self.name]]
-                rc = fn(*lead, _addr(p), _addr(g), *bufs, _addr(s["kahan_comp"]), p.numel(), dt, *scalars, self._stream())
+                rc = fn(*lead, _addr(p), _addr(g), *bufs, _addr(s["kahan_comp"]), p.numel(), DT[p.dtype], *scalars, self._stream())
                 cabi.check(rc, fn.__name__)
 
 
