@@ -15,7 +15,8 @@
  *     argument, or a positive hipError_t value for a HIP runtime failure;
  *     optimi_hip_error_string() explains either.  Nothing throws.
  *   - all buffers are device memory of the current HIP device, contiguous, and of
- *     the one dtype named by `dtype`.  The gradient is never written.
+ *     the one dtype named by `dtype` (the `_multi_mixed` entry points take a dtype per
+ *     tensor).  The gradient is never written.
  *   - work is enqueued on `stream` (a hipStream_t; NULL = the default stream) and
  *     the call returns without waiting for it.
  *   - `kahan_comp` may be NULL whenever the Kahan branch is not taken (fp32 tensors,

@@ -6,6 +6,8 @@ stepping with accumulate-only micro-steps.
 * CPU: the C emulator against the torch for-loop restatement (each pinned by the reference's
   fixtures on the configurations those cover; here they pin each other elsewhere).
 * GPU: the HIP kernels, through the C ABI, against the C emulator.
+* Mixed lists: the same configurations with every other tensor in fp32 beside the 16-bit ones,
+  one launch on the GPU (the ``_multi_mixed`` entry points).
 
 Tensor sizes are multiples of 32 so that ATen's scalar remainder loop (which rounds
 ``add_(x, alpha=...)`` differently from its vector body in low precision) never runs.
@@ -61,11 +63,18 @@ def engine_mode(name, hyper):
     return dict(functional=True) if (name == "adan" and hyper.get("adam_wd")) else {}
 
 
-def draw_tensors(dtype, seed, steps):
+def draw_tensors(dtype, seed, steps, mixed=False):
+    """``mixed``: every other tensor is fp32 instead of ``dtype``."""
     gen = torch.Generator().manual_seed(seed)
-    params = [(torch.randn(n, generator=gen) * 0.02).to(dtype) for n in SIZES]
-    grads = [[(torch.randn(n, generator=gen) * 1e-3 * (1.0, 4.0, 0.25)[t % 3]).to(dtype) for n in SIZES] for t in range(steps)]
+    dts = [torch.float32 if (mixed and i % 2) else dtype for i in range(len(SIZES))]
+    params = [(torch.randn(n, generator=gen) * 0.02).to(d) for n, d in zip(SIZES, dts)]
+    grads = [[(torch.randn(n, generator=gen) * 1e-3 * (1.0, 4.0, 0.25)[t % 3]).to(d) for n, d in zip(SIZES, dts)]
+             for t in range(steps)]
     return params, grads
+
+
+# the whole-list configurations in a 16-bit dtype: the ones a mixed list can be made of
+MIXED_SEEDS = [s for s in range(N_CONFIGS) if draw_config(s)[1] != torch.float32 and not draw_config(s)[3]]
 
 
 def drive(engines, grads, release):
@@ -93,6 +102,32 @@ def test_emulator_matches_forloop(seed):
         G.compare_engines(sca, ref, what, exact=False)
     else:
         G.compare_engines(sca, ref, what, exact=name != "stableadamw")
+
+
+@pytest.mark.parametrize("seed", MIXED_SEEDS)
+def test_emulator_matches_forloop_on_mixed_lists(seed):
+    name, dtype, hyper, _, data_seed = draw_config(seed)
+    torch.set_num_threads(1)
+    params, grads = draw_tensors(dtype, data_seed, 5, mixed=True)
+    mode = engine_mode(name, hyper)
+    sca = ScalarRun(name, [p.clone() for p in params], **mode, **hyper)
+    ref = ForLoopRun(name, [p.clone() for p in params], **mode, **hyper)
+    drive([(sca, torch.clone), (ref, torch.clone)], grads, False)
+    G.compare_engines(sca, ref, f"seed {seed}: {name} {dtype}+fp32 {hyper}", exact=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", MIXED_SEEDS)
+def test_hip_matches_emulator_on_mixed_lists(seed, hip_device):
+    from hip_engine import HipRun
+
+    name, dtype, hyper, _, data_seed = draw_config(seed)
+    params, grads = draw_tensors(dtype, data_seed, 5, mixed=True)
+    mode = engine_mode(name, hyper)
+    hip = HipRun(name, [p.to(hip_device) for p in params], **mode, **hyper)
+    sca = ScalarRun(name, [p.clone() for p in params], **mode, **hyper)
+    drive([(hip, lambda g: g.to(hip_device)), (sca, torch.clone)], grads, False)
+    G.compare_engines(hip, sca, f"seed {seed}: {name} {dtype}+fp32 {hyper}", exact=name != "stableadamw")
 
 
 @pytest.mark.gpu
