@@ -15,6 +15,7 @@ import torch
 
 import golden_util as G
 import optimi_amd
+from optimi_amd import cabi
 from oracle.forloop import ForLoopRun
 
 pytestmark = pytest.mark.gpu
@@ -144,7 +145,8 @@ def test_gradient_release(case, accumulate, dtype, hip_device):
 
 
 def test_two_param_groups_and_mixed_dtypes(hip_device):
-    """A bf16 model with fp32 norm weights in a second, no-decay group: one launch per group and dtype."""
+    """A bf16 model with fp32 norm weights, one of them in the decay group beside the bf16 matrices, the
+    other in a no-decay group of its own: one launch per group, whatever the dtypes in it."""
     torch.manual_seed(0)
     w = [torch.nn.Parameter((torch.randn(300, 70) * 0.02).to(torch.bfloat16).to(hip_device)) for _ in range(3)]
     n = [torch.nn.Parameter(torch.ones(70, device=hip_device)) for _ in range(2)]
@@ -158,7 +160,9 @@ def test_two_param_groups_and_mixed_dtypes(hip_device):
             p.grad = (torch.randn(p.shape, generator=gen) * 1e-3).to(p.dtype).to(hip_device)
         ref_decay.step([p.grad.cpu().clone() for p in w + n[:1]])
         ref_plain.step([p.grad.cpu().clone() for p in n[1:]])
+        before = cabi.lib().optimi_hip_launch_count()
         opt.step()
+        assert cabi.lib().optimi_hip_launch_count() - before == 2, "one kernel launch per parameter group"
         opt.zero_grad()
     for p, q in zip(w + n[:1], ref_decay.params):
         G.assert_close_to_reference(p, q, "decay group", is_param=True)
