@@ -38,6 +38,8 @@ SGD = dict(lr=1e-2, momentum=0.9, weight_decay=1e-2)
 RADAM = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
 
 # name -> (class name, kwargs, dtype, mode, n_steps)
+# dtype "a+b": a parameter group of mixed dtypes - the 2-D tensor has dtype a, the 1-D tensor dtype b
+# (a low-precision weight matrix and an fp32 norm weight, what optimi.utils.to_low_precision leaves behind).
 # mode "group": optimizer.step() on the whole list.
 # mode "release": per-tensor step(param=p) in reverse order, accumulate-only on
 #                 micro-steps where (i+1) % 4 != 0 (optimizer accumulation).
@@ -104,6 +106,14 @@ CASES = {
     "adan_bf16_kahan_adamwd_declr_functional_release": (
         "Adan", dict(ADAN, adam_wd=True, kahan_sum=True, decouple_lr=True, weight_decay=1e-3, max_lr=2e-3),
         "bfloat16", "functional_release", 8),
+    # one parameter group holding a 16-bit matrix and an fp32 vector: the group's Kahan flag comes on because of the
+    # former (optimi/adam.py:100-102) and must not touch the latter
+    "adamw_mixed_bf16_fp32": ("AdamW", dict(ADAMW), "bfloat16+float32", "group", 10),
+    "adamw_mixed_bf16_fp32_release": ("AdamW", dict(ADAMW), "bfloat16+float32", "release", 8),
+    "lion_mixed_fp16_fp32": ("Lion", dict(LION), "float16+float32", "group", 10),
+    "stableadamw_mixed_bf16_fp32_declr": ("StableAdamW", dict(SADAMW, weight_decay=1e-3, decouple_lr=True, max_lr=2e-3), "bfloat16+float32", "group", 10),
+    "adan_mixed_bf16_fp32_kahan": ("Adan", dict(ADAN, kahan_sum=True), "bfloat16+float32", "group", 10),
+    "ranger_mixed_bf16_fp32": ("Ranger", dict(RADAM, k=3), "bfloat16+float32", "group", 10),
 }
 
 # The seed each committed fixture's inputs were drawn with.  Literal, so that adding a case can
@@ -126,6 +136,8 @@ SEEDS = {
     "stableadamw_fp16_kahan": 1028, "stableadamw_fp32": 1024,
     "adan_fp32_adamwd_functional": 3001, "adan_bf16_plain_adamwd_functional": 3002,
     "adan_bf16_kahan_adamwd_functional": 3003, "adan_bf16_kahan_adamwd_declr_functional_release": 3004,
+    "adamw_mixed_bf16_fp32": 4001, "adamw_mixed_bf16_fp32_release": 4002, "lion_mixed_fp16_fp32": 4003,
+    "stableadamw_mixed_bf16_fp32_declr": 4004, "adan_mixed_bf16_fp32_kahan": 4005, "ranger_mixed_bf16_fp32": 4006,
 }
 
 
@@ -148,20 +160,28 @@ def grad_scale(step: int) -> float:
     return 1e-3 * (1.0, 1.0, 4.0, 0.5, 2.0)[step % 5]
 
 
-def make_inputs(dtype: torch.dtype, n_steps: int, seed: int):
+def case_dtypes(dtype_name: str) -> list[torch.dtype]:
+    """The dtype of every tensor of a case: "bfloat16" -> all bf16, "bfloat16+float32" -> one each."""
+    names = dtype_name.split("+")
+    return [getattr(torch, names[i % len(names)]) for i in range(len(SHAPES))]
+
+
+def make_inputs(dtype, n_steps: int, seed: int):
+    """``dtype``: one torch dtype for every tensor, or a list with one per tensor."""
+    dtypes = list(dtype) if isinstance(dtype, (list, tuple)) else [dtype] * len(SHAPES)
     gen = torch.Generator().manual_seed(seed)
     params, grads = [], []
-    for shape in SHAPES:
+    for shape, dt in zip(SHAPES, dtypes):
         p = torch.randn(shape, generator=gen) * 0.02
         p.view(-1)[:2] = torch.tensor([0.0, 1.0])
-        params.append(p.to(dtype))
+        params.append(p.to(dt))
     for t in range(n_steps):
         gs = []
-        for shape in SHAPES:
+        for shape, dt in zip(SHAPES, dtypes):
             g = torch.randn(shape, generator=gen) * grad_scale(t)
             # special values: zero, below eps, large, and a sign flip partner
             g.view(-1)[:6] = torch.tensor([0.0, 1e-9, -1e-9, 1.0, -0.5, 3e-7])
-            gs.append(g.to(dtype))
+            gs.append(g.to(dt))
         grads.append(gs)
     return params, grads
 
@@ -177,8 +197,7 @@ def snapshot(out: dict, tag: str, params, opt):
 
 def run_case(optimi, name: str, seed: int) -> dict:
     cls_name, kwargs, dtype_name, mode, n_steps = CASES[name]
-    dtype = getattr(torch, dtype_name)
-    p0, grads = make_inputs(dtype, n_steps, seed)
+    p0, grads = make_inputs(case_dtypes(dtype_name), n_steps, seed)
     out = {}
     for i, p in enumerate(p0):
         out[f"in.param.{i}"] = to_np(p)

@@ -24,6 +24,7 @@ _spec.loader.exec_module(_mk)
 CASES = _mk.CASES
 SEEDS = _mk.SEEDS
 make_inputs = _mk.make_inputs
+case_dtypes = _mk.case_dtypes
 STATE_KEYS = _mk.STATE_KEYS
 N_TENSORS = len(_mk.SHAPES)
 
@@ -31,17 +32,18 @@ OPT_NAME = {"Adam": "adam", "AdamW": "adamw", "Lion": "lion", "StableAdamW": "st
             "SGD": "sgd", "RAdam": "radam", "Ranger": "ranger"}
 
 
-def torch_tail(name: str, numel: int) -> int:
-    """How many trailing elements of a bf16 tensor of a fixture case to leave out when comparing
+def torch_tail(name: str, numel: int, dtype: torch.dtype | None = None) -> int:
+    """How many trailing elements of a bf16 or fp16 tensor (``dtype``; by default the dtype of the
+    case) of a fixture case to leave out when comparing
     against anything but torch itself.  ATen's CPU ``add_(other, alpha=...)`` fuses
     ``self + alpha*other`` in fp32 in its vector body but works in bf16 arithmetic (the product
     rounded on its own) in the scalar loop over the last ``numel % 32`` elements, so the
     reference's own output is not uniform there.  SGD (``p += -lr*m``), RAdam/Ranger before
     rectification, Ranger's Lookahead and L2 weight decay go through that op; the kernels and
     the C emulator follow the vector body everywhere."""
-    dtype = CASES[name][2]
+    low = CASES[name][2] in ("bfloat16", "float16") if dtype is None else dtype in (torch.bfloat16, torch.float16)
     uses_add_alpha = name.split("_")[0] in ("sgd", "radam", "ranger") or name.endswith("_l2")
-    return numel % 32 if (dtype in ("bfloat16", "float16") and uses_add_alpha) else 0
+    return numel % 32 if (low and uses_add_alpha) else 0
 
 
 def case_names(functional: bool | None = None):

@@ -29,7 +29,7 @@ FP32_FLOOR_PARAM = 1e-2
 
 
 def compare_snapshot(name, key, got, want, param_want=None):
-    keep = want.numel() - G.torch_tail(name, want.numel())  # see golden_util.torch_tail
+    keep = want.numel() - G.torch_tail(name, want.numel(), want.dtype)  # see golden_util.torch_tail
     got, want = got.flatten()[:keep], want.flatten()[:keep]
     if param_want is not None:
         param_want = param_want.flatten()[:keep]

@@ -8,6 +8,8 @@ What is compared with what:
   loops over the tensors of a group whatever their dtypes): the tolerance of the one-dtype tests;
 * the launch counter: one kernel per step (three for StableAdamW), where the one-dtype entry
   points need two (six).
+The reference's own output for a group of mixed dtypes is held by the ``*_mixed_*`` fixtures
+(``tests/test_hip_golden.py`` replays them through the same entry points).
 """
 
 import types

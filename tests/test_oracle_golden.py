@@ -41,7 +41,7 @@ def test_scalar_emulator(name):
     assert sorted(out) == wanted
     for k in wanted:
         got, want = out[k].flatten(), fx[k].flatten()
-        keep = want.numel() - G.torch_tail(name, want.numel())
+        keep = want.numel() - G.torch_tail(name, want.numel(), want.dtype)
         got, want = got[:keep], want[:keep]
         if want.dtype != torch.float32 or not (".param." in k or ".la_param." in k):
             n_bad = int(((bits(got) != bits(want)) & ~(got.isnan() & want.isnan())).sum())
@@ -58,7 +58,7 @@ def test_committed_recipe_regenerates_the_fixture_inputs(name):
     need the reference; the inputs do not)."""
     _cls, _kwargs, dtype_name, _mode, n_steps = G.CASES[name]
     fx = G.load(name)
-    params, grads = G.make_inputs(getattr(torch, dtype_name), n_steps, G.SEEDS[name])
+    params, grads = G.make_inputs(G.case_dtypes(dtype_name), n_steps, G.SEEDS[name])
     stored = sorted(k for k in fx if k.startswith("in."))
     assert len(stored) == len(params) * (1 + n_steps)
     for i, p in enumerate(params):
