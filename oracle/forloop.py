@@ -33,6 +33,8 @@ function                   pinned by
                            restatement; scalar C emulator
 functional ``adam`` …      golden fixtures (class API and gradient-release /
                            accumulation runs of the reference)
+``ForLoopRun`` on a group  golden fixtures of one parameter group holding a
+of mixed dtypes            16-bit and an fp32 tensor (``*_mixed_*``)
 =========================  ====================================================
 """
 
