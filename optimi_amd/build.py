@@ -55,7 +55,7 @@ def build_lib(verbose: bool = False) -> str:
     return LIB_PATH
 
 
-def build_binding(verbose: bool = False) -> str:
+def _binding_commands():
     import torch
     from torch.utils import cpp_extension as ce
 
@@ -63,23 +63,56 @@ def build_binding(verbose: bool = False) -> str:
                                                      f"-I{sysconfig.get_paths()['include']}"]
     torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
     abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
-    cmd = [
-        shutil.which("g++") or "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-deprecated-declarations",
+    gxx = shutil.which("g++") or "g++"
+    obj = os.path.join(CSRC, "torch_binding.o")
+    compile_cmd = [
+        gxx, "-O2", "-std=c++17", "-fPIC", "-c", "-Wno-deprecated-declarations",
         "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H",
-        f"-D_GLIBCXX_USE_CXX11_ABI={abi}", *inc, os.path.join(CSRC, "torch_binding.cpp"), "-o", BINDING_PATH,
+        f"-D_GLIBCXX_USE_CXX11_ABI={abi}", *inc, os.path.join(CSRC, "torch_binding.cpp"), "-o", obj,
+    ]
+    link_cmd = [
+        gxx, "-shared", obj, "-o", BINDING_PATH,
         f"-L{HERE}", "-loptimi_hip", f"-L{torch_lib}", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip",
         "-ltorch_python", f"-L{ROCM_HOME}/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}",
         f"-Wl,-rpath,{ROCM_HOME}/lib",
     ]
-    if verbose:
-        print(" ".join(cmd))
-    _run(cmd)
+    return compile_cmd, link_cmd, obj
+
+
+def build_binding(verbose: bool = False) -> str:
+    """Compiles and links the binding; the kernel library must exist already (it is linked against)."""
+    compile_cmd, link_cmd, obj = _binding_commands()
+    try:
+        for cmd in (compile_cmd, link_cmd):
+            if verbose:
+                print(" ".join(cmd))
+            _run(cmd)
+    finally:
+        if os.path.exists(obj):
+            os.remove(obj)
     return BINDING_PATH
 
 
 def build_all(verbose: bool = False):
-    build_lib(verbose)
-    build_binding(verbose)
+    """Both pieces; the binding's translation unit compiles while hipcc works on the kernels,
+    and is linked once the library it links against is there."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    compile_cmd, link_cmd, obj = _binding_commands()
+    try:
+        with ThreadPoolExecutor(max_workers=2) as pool:
+            lib = pool.submit(build_lib, verbose)
+            if verbose:
+                print(" ".join(compile_cmd))
+            binding = pool.submit(_run, compile_cmd)
+            lib.result()
+            binding.result()
+        if verbose:
+            print(" ".join(link_cmd))
+        _run(link_cmd)
+    finally:
+        if os.path.exists(obj):
+            os.remove(obj)
 
 
 if __name__ == "__main__":
