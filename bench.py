@@ -93,6 +93,9 @@ MEASURED_TRAFFIC = {
     "stableadamw_bf16_kahan_llama7b": (1.4887e11, "profiles/lion_stableadamw_adan_adamw1b_hbm_traffic.txt"),
     "adan_bf16_kahan_llama7b": (1.7524e11, "profiles/lion_stableadamw_adan_adamw1b_hbm_traffic.txt"),
     "adamw_bf16_kahan_declr_llama1b": (2.170e10, "profiles/lion_stableadamw_adan_adamw1b_hbm_traffic.txt"),
+    "adamw_bf16_kahan_fp32_embeddings_norms_llama7b": (1.23964e11, "profiles/adamw_mixed_dtype_and_fp32_lists_hbm_traffic.txt"),
+    "adamw_fp32_llama1b": (3.3754e10, "profiles/adamw_mixed_dtype_and_fp32_lists_hbm_traffic.txt"),
+    "adamw_fp32_mlp": (4.701e8, "profiles/adamw_mixed_dtype_and_fp32_lists_hbm_traffic.txt"),
 }
 
 # the benchmark configurations reported under "extra" next to the headline workload
