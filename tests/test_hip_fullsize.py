@@ -7,6 +7,8 @@
   covers all five distinct shapes is also stepped through the per-tensor entry point from cloned
   inputs – a whole-list launch must equal per-tensor launches bit for bit, whatever the list size.
   The same sample is checked against the C emulator on the CPU (10 steps).
+* the same 7B list with fp32 embeddings and norm weights beside bf16 + Kahan (AdamW, StableAdamW): one launch
+  over both dtypes equals per-tensor launches bit for bit.
 * C5 – AdamW bf16 + Kahan per tensor in reverse order with ``accumulation_steps=4`` on the 7B shapes
   sample, and the 10,000-tensor stress list (sizes log-uniform in [128, 65536]) both as one launch and
   as 10,000 per-tensor launches, against the C emulator.
@@ -100,6 +102,48 @@ def test_c3_c4_llama7b_whole_list_equals_per_tensor(name, hip_device):
         whole.step(grads)
         del grads
     torch.cuda.synchronize()
+    for j, i in enumerate(SAMPLE_7B):
+        G.assert_bits_equal(whole.params[i], sample.params[j], f"{name} tensor {i} param")
+        for key in G.STATE_KEYS:
+            a = whole.state[i].get(key)
+            if a is not None:
+                G.assert_bits_equal(a, sample.state[j][key], f"{name} tensor {i} {key}")
+    del whole, sample, params
+    free()
+
+
+@pytest.mark.parametrize("name", ["adamw", "stableadamw"])
+def test_llama7b_list_of_mixed_dtypes_equals_per_tensor(name, hip_device):
+    """The 7B list with its embeddings and norm weights in fp32 (262 M parameters, two of the tensors
+    past 2^27 elements) beside bf16 + Kahan: one launch over both dtypes against per-tensor launches
+    of each tensor's own dtype, bit for bit - 13.7 M workgroups, chunks of 8192 and of 4096 elements
+    in one grid."""
+    from hip_engine import HipRun
+
+    from optimi_amd import cabi
+
+    shapes = llama_shapes(4096, 11008, 32)
+    hyper = HYPER[name]
+    gen = torch.Generator(device=hip_device).manual_seed(7)
+    params = draw(shapes, hip_device, gen, 0.02, ones_for_1d=True)
+    fp32 = [i for i, s in enumerate(shapes) if len(s) == 1 or s[0] == 32000]
+    assert len(fp32) == 66 and sum(math.prod(shapes[i]) for i in fp32) == 262_406_144
+    for i in fp32:
+        params[i] = params[i].float()
+    sample = HipRun(name, [params[i].clone() for i in SAMPLE_7B], gradient_release=True, **hyper)
+    whole = HipRun(name, params, **hyper)
+    for _ in range(2):
+        grads = draw(shapes, hip_device, gen, 1e-3)
+        for i in fp32:
+            grads[i] = grads[i].float()
+        for j, i in enumerate(SAMPLE_7B):
+            sample.step_param(j, grads[i].clone())
+        before = cabi.lib().optimi_hip_launch_count()
+        whole.step(grads)
+        assert cabi.lib().optimi_hip_launch_count() - before == (3 if name == "stableadamw" else 1)
+        del grads
+    torch.cuda.synchronize()
+    assert {whole.params[i].dtype for i in SAMPLE_7B} == {torch.bfloat16, torch.float32}
     for j, i in enumerate(SAMPLE_7B):
         G.assert_bits_equal(whole.params[i], sample.params[j], f"{name} tensor {i} param")
         for key in G.STATE_KEYS:
