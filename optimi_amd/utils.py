@@ -27,7 +27,7 @@ def param_groups_weight_decay(model: nn.Module, weight_decay: float = 1e-2,
                               additional_layers: Iterable[str] | None = None) -> list[dict[str, Any]]:
     """Two parameter groups: biases, 0-d/1-d tensors (normalization weights) and any parameter
     whose name contains one of ``additional_layers`` get ``weight_decay=0``; all other trainable
-    parameters get ``weight_decay``.  Each group is stepped as one launch per dtype.
+    parameters get ``weight_decay``.  Each group is stepped as one launch, whatever dtypes it holds.
     (optimi/utils.py:41-71; order of the groups as there: no-decay first.)"""
     skip = tuple(additional_layers) if additional_layers is not None else ()
     groups = {False: [], True: []}
@@ -62,8 +62,8 @@ def to_low_precision(model: nn.Module, dtype: torch.dtype = torch.bfloat16, devi
       "rope", "rotary"), or that are instances of a module type listed there, keep their own
       buffers in float32 (their parameters are cast).
 
-    Non-floating-point tensors are left alone.  The optimizers step the resulting mixed
-    bf16 / fp32 parameter groups as one launch per dtype.  (optimi/utils.py:104-169)"""
+    Non-floating-point tensors are left alone.  The optimizers step each of the resulting mixed
+    bf16 / fp32 parameter groups as one launch.  (optimi/utils.py:104-169)"""
     mod_types = _as_tuple(fp32_modules)
     if not all(_is_module_type(t) for t in mod_types):
         raise TypeError("fp32_modules must be nn.Module subclass type(s)")
