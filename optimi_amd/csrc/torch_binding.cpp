@@ -537,9 +537,10 @@ void check_hip(hipError_t err, const char* what) {
 // Parks the steps of small tensors and launches them together, as one list per run of steps
 // that share everything but their tensors (optimizer, device, stream, flags and every scalar -
 // which includes the step count through the debiased betas; fp32 tensors and tensors of one
-// 16-bit dtype share a list, so a bf16 model with fp32 norms does not break the run at every norm).  A tensor of a few
-// thousand elements costs far more to launch than to update, so a model with thousands of
-// them is bound by launches; one list launch replaces up to `max_tensors` of them.  The queue
+// 16-bit dtype share a list, so a bf16 model with fp32 norms does not break the run at every
+// norm).  A tensor of a few thousand elements costs far more to launch than to update, so a
+// model with thousands of them is bound by launches; one list launch replaces up to
+// `max_tensors` of them.  The queue
 // keeps each parked gradient alive until its launch; `max_total` bounds how many bytes of
 // gradients that may be.  Results are those of the per-tensor launches, bit for bit.
 //
