@@ -692,14 +692,14 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
 // embeddings or norms stay fp32): every workgroup looks its tensor up as above and runs that
 // dtype's step on its tile, with that dtype's scalars.  Chunks are kChunkBytes per array for
 // both, so the grid does not care which is which.
-template <class OpLow, class OpF32>
+template <class OpLow, class OpF32, bool MULTI>
 __global__ void __launch_bounds__(kThreads)
-mixed_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, typename OpLow::Scalars s_low,
-             typename OpF32::Scalars s_f32, double* __restrict__ partials) {
+mixed_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, const FewTable few,
+             typename OpLow::Scalars s_low, typename OpF32::Scalars s_f32, double* __restrict__ partials) {
   const int64_t chunk_id = blockIdx.x / kSub;
   const int sub = blockIdx.x % kSub;
-  const int tensor = chunk_map[chunk_id];
-  const TensorEntry& e = table[tensor];
+  const int tensor = MULTI ? chunk_map[chunk_id] : optimi_tables::few_lookup(few, chunk_id);
+  const TensorEntry& e = MULTI ? table[tensor] : few.e[tensor];
   if (e.flags & optimi_tables::kEntryF32) tile_step<OpF32>(e, tensor, chunk_id, sub, s_f32, partials);
   else tile_step<OpLow>(e, tensor, chunk_id, sub, s_low, partials);
 }
@@ -884,7 +884,7 @@ struct ListPlan {
   int n_tensors = 0;
   int64_t n_chunks = 0;
   bool resident = false;      // the list's arrays fit the last-level cache and were touched recently
-  bool mixed = false;         // fp32 tensors beside 16-bit ones (always through the device tables)
+  bool mixed = false;         // fp32 tensors beside 16-bit ones
 };
 
 constexpr int64_t kMaxChunks = (int64_t)0x7fffffff / kSub;  // the grid is chunks x kSub workgroups
@@ -908,8 +908,8 @@ int list_dtypes(int n_tensors, const int* dtypes, int* low, bool* mixed) {
 }
 
 // Validates the list and gets its tables to where the kernel reads them: into `plan` itself for
-// a list of at most kFew tensors of one dtype (nothing is uploaded), else into the group's device
-// tables, (re)building the chunk map and tensor table and uploading what changed.
+// a list of at most kFew tensors (nothing is uploaded), else into the group's device tables,
+// (re)building the chunk map and tensor table and uploading what changed.
 // `lists[a]` may be nullptr for an array the launch does not touch (`need` has its bit clear).
 // `dtypes`: nullptr when every tensor has `dtype`; else every tensor's own dtype, `dtype` being
 // the 16-bit one among them, and fp32 tensors have no array in `low_precision_only`.
@@ -925,7 +925,7 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
 
   plan->n_tensors = n_tensors;
   plan->mixed = dtypes != nullptr;
-  plan->few = n_tensors <= kFew && !plan->mixed;
+  plan->few = n_tensors <= kFew;
   std::memset(&plan->table, 0, sizeof(plan->table));
   std::vector<TensorEntry> fresh;
   TensorEntry* entries = plan->table.e;
@@ -1107,8 +1107,12 @@ void launch_list(optimi_group* g, const ListPlan& plan, const typename Op::Scala
   ++kernel_launches;
   if constexpr (!std::is_same<typename Op::DT, F32>::value) {
     if (plan.mixed) {
-      mixed_kernel<Op, typename Op::F32Partner><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
-          (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, s, *s_f32, partials);
+      if (plan.few)
+        mixed_kernel<Op, typename Op::F32Partner, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
+            nullptr, nullptr, plan.table, s, *s_f32, partials);
+      else
+        mixed_kernel<Op, typename Op::F32Partner, true><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
+            (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, *s_f32, partials);
       return;
     }
   }

@@ -27,11 +27,13 @@ pytestmark = pytest.mark.gpu
 # 4096 elements, a 16-bit one 8192), empty tensors at the start, in the middle and at the end
 SIZES = [0, 8193, 5, 4096, 4097, 0, 513, 8192, 1, 20001, 1024, 12288, 7, 100003, 64, 0]
 F32_AT = {1, 2, 5, 6, 9, 11, 13, 15}  # positions of the fp32 tensors: both kinds begin, end and neighbour each other
+# 16 tensors travel as a kernel argument; four more and the list goes through the device tables
+MORE_SIZES, MORE_F32_AT = [700, 12288, 0, 33], {17, 19}
 
 
-def draw_mixed(low, steps, seed):
-    params, grads = draw(SIZES, torch.float32, steps, seed)
-    dt = [torch.float32 if i in F32_AT else low for i in range(len(SIZES))]
+def draw_mixed(low, steps, seed, sizes=SIZES, f32_at=F32_AT):
+    params, grads = draw(sizes, torch.float32, steps, seed)
+    dt = [torch.float32 if i in f32_at else low for i in range(len(sizes))]
     return [p.to(d) for p, d in zip(params, dt)], [[g.to(d) for g, d in zip(gs, dt)] for gs in grads]
 
 
@@ -56,18 +58,20 @@ def launches():
     return cabi.lib().optimi_hip_launch_count()
 
 
+@pytest.mark.parametrize("tables", ["kernel_argument", "device"])
 @pytest.mark.parametrize("low,kahan", [(torch.bfloat16, None), (torch.bfloat16, False), (torch.float16, None)],
                          ids=["bf16_kahan", "bf16_plain", "fp16_kahan"])
 @pytest.mark.parametrize("cfg", list(CONFIGS))
-def test_mixed_list_is_one_launch_with_the_bits_of_two(cfg, low, kahan, hip_device):
+def test_mixed_list_is_one_launch_with_the_bits_of_two(cfg, low, kahan, tables, hip_device):
     hyper = dict(CONFIGS[cfg])
     if kahan is False:
         hyper["kahan_sum"] = False
     name = OPT_OF[cfg]
     steps = 6
-    params, grads = draw_mixed(low, steps, seed=sum(map(ord, cfg)) + 1)
-    idx_f32 = sorted(F32_AT)
-    idx_low = [i for i in range(len(SIZES)) if i not in F32_AT]
+    sizes, f32_at = (SIZES, F32_AT) if tables == "kernel_argument" else (SIZES + MORE_SIZES, F32_AT | MORE_F32_AT)
+    params, grads = draw_mixed(low, steps, seed=sum(map(ord, cfg)) + 1, sizes=sizes, f32_at=f32_at)
+    idx_f32 = sorted(f32_at)
+    idx_low = [i for i in range(len(sizes)) if i not in f32_at]
     pick = lambda col, idx: [col[i] for i in idx]  # noqa: E731
     torch.set_num_threads(1)
     guard = Guarded(hip_device)
@@ -91,7 +95,7 @@ def test_mixed_list_is_one_launch_with_the_bits_of_two(cfg, low, kahan, hip_devi
     for t, n in enumerate(per_step):
         want = (plain_sgd_accumulate if t == 2 else 1) if name != "stableadamw" else (1 if t == 2 else 3)
         assert n == want, f"{cfg} step {t}: {n} kernel launches for the mixed list, expected {want}"
-    G.compare_engines(mixed, split_view(only_low, idx_low, only_f32, idx_f32, len(SIZES)), f"{cfg} mixed-vs-split", exact=True)
+    G.compare_engines(mixed, split_view(only_low, idx_low, only_f32, idx_f32, len(sizes)), f"{cfg} mixed-vs-split", exact=True)
     tail = 32 if cfg in ADD_ALPHA else 0
     G.compare_engines(mixed, ref, f"{cfg} mixed-vs-forloop", exact=False, body_only=tail)
 
