@@ -273,8 +273,9 @@ int optimi_hip_ranger_single(void* param, const void* grad, void* exp_avg, void*
  * ------------------------------------------------------------------------------- */
 int optimi_hip_copy_probe(void* dst, const void* src, int64_t bytes, optimi_stream_t stream);
 
-/* Measurement aid (no counterpart in the reference): the number of kernels this library has
- * launched in this process so far, every entry point and every thread counted.  Tests and
+/* Measurement aid (no counterpart in the reference): the number of step, reduction and probe
+ * kernels this library has launched in this process so far, every entry point and every thread
+ * counted (the small copy that brings a changed tensor table to the device is not).  Tests and
  * benchmarks take differences of it to see how many launches a step costs. */
 int64_t optimi_hip_launch_count(void);
 
