@@ -484,3 +484,38 @@ def test_foreach_true_selects_the_hip_kernels(hip_device):
         warnings.simplefilter("ignore")
         opt = optimi_amd.AdamW(a.parameters(), lr=1e-3, foreach=True, gradient_release=True)
     assert opt.param_groups[0]["foreach"] is False
+
+
+def test_add_param_group_after_steps(hip_device):
+    """A group added later (layers unfrozen during fine-tuning) starts its own step counter at zero
+    (optimi/adam.py:132-134: the counter is created at the group's first step) and takes the
+    constructor's defaults for what it does not set."""
+    torch.manual_seed(3)
+    a = [torch.nn.Parameter((torch.randn(130, 40) * 0.02).to(torch.bfloat16).to(hip_device)) for _ in range(2)]
+    b = [torch.nn.Parameter((torch.randn(77) * 0.02).to(hip_device))]
+    hyper = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6)
+    opt = optimi_amd.AdamW(a, weight_decay=1e-2, **hyper)
+    ref_a = ForLoopRun("adamw", [p.detach().cpu().clone() for p in a], weight_decay=1e-2, **hyper)
+    ref_b = ForLoopRun("adamw", [p.detach().cpu().clone() for p in b], weight_decay=0.0, **hyper)
+    gen = torch.Generator().manual_seed(4)
+
+    def grads_for(ps):
+        for p in ps:
+            p.grad = (torch.randn(p.shape, generator=gen) * 1e-3).to(p.dtype).to(hip_device)
+        return [p.grad.cpu().clone() for p in ps]
+
+    for _ in range(3):
+        ref_a.step(grads_for(a))
+        opt.step()
+        opt.zero_grad()
+    opt.add_param_group({"params": b, "weight_decay": 0.0})
+    for _ in range(4):
+        ga, gb = grads_for(a), grads_for(b)
+        ref_a.step(ga)
+        ref_b.step(gb)
+        opt.step()
+        opt.zero_grad()
+    assert int(opt.param_groups[0]["step"]) == 7 and int(opt.param_groups[1]["step"]) == 4
+    for p, q in zip(a, ref_a.params):
+        G.assert_close_to_reference(p, q, "first group", is_param=True)
+    G.assert_close_to_reference(b[0], ref_b.params[0], "group added later", is_param=True)
