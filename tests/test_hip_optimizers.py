@@ -488,7 +488,7 @@ def test_foreach_true_selects_the_hip_kernels(hip_device):
 
 def test_add_param_group_after_steps(hip_device):
     """A group added later (layers unfrozen during fine-tuning) starts its own step counter at zero
-    (optimi/adam.py:132-134: the counter is created at the group's first step) and takes the
+    (optimi/adam.py:134-136: the counter is created at the group's first step) and takes the
     constructor's defaults for what it does not set."""
     torch.manual_seed(3)
     a = [torch.nn.Parameter((torch.randn(130, 40) * 0.02).to(torch.bfloat16).to(hip_device)) for _ in range(2)]
