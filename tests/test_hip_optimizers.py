@@ -519,3 +519,34 @@ def test_add_param_group_after_steps(hip_device):
     for p, q in zip(a, ref_a.params):
         G.assert_close_to_reference(p, q, "first group", is_param=True)
     G.assert_close_to_reference(b[0], ref_b.params[0], "group added later", is_param=True)
+
+
+@pytest.mark.parametrize("case", list(CASES))
+def test_mixed_group_with_state_dict_roundtrip(case, hip_device):
+    """One parameter group of bf16 matrices and fp32 vectors (what ``to_low_precision`` leaves
+    behind), checkpointed into a fresh optimizer twice on the way: states of both dtypes, the
+    1-element Kahan placeholders of the fp32 tensors and the group's step counter survive, and
+    every tensor keeps following the reference's for-loop path."""
+    cls, oname, hyper = CASES[case]
+    gen = torch.Generator().manual_seed(9)
+    shapes = [(96, 64), (64,), (200, 32), (32,)]
+    params = [torch.nn.Parameter((torch.randn(s, generator=gen) * 0.02).to(torch.bfloat16 if len(s) == 2 else torch.float32)
+                                 .to(hip_device)) for s in shapes]
+    opt = cls(params, **hyper)
+    ref = oracle_for(oname, params, hyper)
+    for it in range(10):
+        for p in params:
+            p.grad = (torch.randn(p.shape, generator=gen) * 1e-3).to(p.dtype).to(hip_device)
+        grads = [p.grad.detach().cpu().clone() for p in params]
+        opt.step()
+        opt.zero_grad()
+        ref.step(grads)
+        compare(opt, params, ref, f"{case} mixed it {it}")
+        if it in (2, 6):
+            blob = io.BytesIO()
+            torch.save(opt.state_dict(), blob)
+            blob.seek(0)
+            fresh = cls(params, **hyper)
+            fresh.load_state_dict(torch.load(blob, weights_only=True))
+            opt = fresh
+    assert opt.state[params[0]]["exp_avg"].dtype == torch.bfloat16 and opt.state[params[1]]["exp_avg"].dtype == torch.float32
