@@ -271,39 +271,37 @@ struct RangerScalars {
   float alpha_d;
 };
 
-// Ranger = the RAdam step, then every k-th step a Lookahead sync with the slow weights.
+// Ranger = the RAdam step, then every k-th step (step % k == 0) a Lookahead sync with the slow
+// weights.  This Op is such a synchronising step; every other Ranger step is RAdam's Op.
 // slots: 0 param, 1 grad, 2 exp_avg, 3 exp_avg_sq, 4 kahan_comp, 5 la_param   optimi/ranger.py:402-473
-// LA: this step synchronises (step % k == 0)
-template <class DT_, bool KAHAN, bool UPDATE, int WD, int TAIL, bool LA>
+template <class DT_, bool KAHAN, int WD, int TAIL>
 struct RangerOp {
   using DT = DT_;
-  using F32Partner = RangerOp<F32, false, UPDATE, WD, TAIL, LA>;
+  using F32Partner = RangerOp<F32, false, WD, TAIL>;
   using Scalars = RangerScalars;
-  using Inner = AdamTailOp<DT_, KAHAN, UPDATE, WD, TAIL>;
+  using Inner = AdamTailOp<DT_, KAHAN, true, WD, TAIL>;
   static constexpr int kArrays = 6;
-  static constexpr uint32_t kLoad = Inner::kLoad | ((UPDATE && LA) ? bit(5) : 0);
-  static constexpr uint32_t kStore = Inner::kStore | ((UPDATE && LA) ? bit(5) : 0);
+  static constexpr uint32_t kLoad = Inner::kLoad | bit(5);
+  static constexpr uint32_t kStore = Inner::kStore | bit(5);
   static constexpr bool kReduce = false;
   __device__ static __forceinline__ void prepare(Scalars&, int) {}
   __device__ static __forceinline__ void elem(f32x2* x, const Scalars& s, f32x2& q) {
     Inner::elem(x, s.a, q);
-    if (UPDATE && LA) {
-      f32x2 p = x[0], la = x[5];
-      f32x2 t = DT::R2(p - la);
-      if (KAHAN) {
-        f32x2 k = x[4];
-        k = DT::R2(fma2(t, splat(s.alpha_d), k));
-        f32x2 old = la;
-        la = DT::R2(old + k);
-        f32x2 err = DT::R2(old - la);
-        k = DT::R2(fma2(err, splat(s.alpha_d), k));
-        x[4] = k;
-      } else {
-        la = DT::R2(fma2(t, splat(s.alpha_d), la));
-      }
-      x[0] = la;
-      x[5] = la;
+    f32x2 p = x[0], la = x[5];
+    f32x2 t = DT::R2(p - la);
+    if (KAHAN) {
+      f32x2 k = x[4];
+      k = DT::R2(fma2(t, splat(s.alpha_d), k));
+      f32x2 old = la;
+      la = DT::R2(old + k);
+      f32x2 err = DT::R2(old - la);
+      k = DT::R2(fma2(err, splat(s.alpha_d), k));
+      x[4] = k;
+    } else {
+      la = DT::R2(fma2(t, splat(s.alpha_d), la));
     }
+    x[0] = la;
+    x[5] = la;
   }
 };
 
@@ -1037,9 +1035,10 @@ int finish_list(optimi_group* g, const ListPlan& plan, hipStream_t stream) {
 // workgroups; reachable occupancies are therefore 32, 25, 21, 18, 16, 14, 12, 11, 10, 9, 8, ...
 // The table holds the measured optimum in granules on MI355X with the write-through tile stores
 // (7B-parameter lists; 5 streams = StableAdamW pass 1 and accumulate-only Adam, 6 = pass 2,
-// 7 = Lion / SGD and fp32 Adam, 9 = Adam with Kahan, 13 = Adan; entries in between are
-// interpolated).  fp32 Adan (11 streams) does best at 17 granules, 7 workgroups (a Llama-1B-shaped
-// list: 8.12 ms at 16, 7.98 ms at 17 and 18).  16-bit list launches of fewer than kLongLaunch
+// 7 = Lion / SGD and fp32 Adam, 9 = Adam with Kahan, 11 = Ranger's Lookahead step and Adan without
+// Kahan (22.75 ms at 12 granules against 23.34 at 14, and 23.46 against 23.80), 13 = Adan; entries
+// in between are interpolated).  fp32 Adan (also 11 streams) does best at 17 granules, 7
+// workgroups (a Llama-1B-shaped list: 8.12 ms at 16, 7.98 ms at 17 and 18).  16-bit list launches of fewer than kLongLaunch
 // workgroups (the Llama-1B-shaped list) do best one granule lower, i.e. with one more workgroup
 // resident.  Lists that live in the last-level cache follow the same table (16.8 M parameters:
 // fp32 AdamW 68.9 us at 6 granules, 67.5 us at 10 and 11; bf16 AdamW 48.7 us at 6, 47.0 us at 12;
@@ -1047,7 +1046,7 @@ int finish_list(optimi_group* g, const ListPlan& plan, hipStream_t stream) {
 // per CU for every kernel (nearest reachable count at or above it; 0 = no throttle); read once.
 constexpr int kLdsGranule = 1280, kLdsGranules = 128;
 constexpr int kMaxStreams = 2 * kMaxArrays;
-constexpr int kBestGranules[kMaxStreams + 1] = {4, 4, 4, 4, 6, 8, 8, 11, 11, 12, 13, 14, 16, 16, 16};
+constexpr int kBestGranules[kMaxStreams + 1] = {4, 4, 4, 4, 6, 8, 8, 11, 11, 12, 12, 12, 14, 16, 16};
 constexpr int64_t kLongLaunch = (int64_t)1 << 22;  // workgroups
 
 int forced_waves() {
@@ -1306,18 +1305,18 @@ void sgd_dispatch(int dtype, bool kahan, bool update, int wd, int mom, Launch&& 
   });
 }
 
-// Launches the Ranger variant: ... x rectified or not x Lookahead step or not.
+// Launches the Ranger variant of a step that synchronises with the slow weights: ... x rectified
+// or not.  (A Ranger step without the Lookahead sync, and every accumulate-only one, is the RAdam
+// step - optimi/ranger.py:402-473 - and runs RAdam's kernels.)
 template <class Launch>
-void ranger_dispatch(int dtype, bool kahan, bool update, int wd, bool rectify, bool la, Launch&& launch) {
-  dispatch_tags(dtype, kahan, update, wd, [&](auto dt, auto kh, auto up, auto w) {
+void ranger_dispatch(int dtype, bool kahan, int wd, bool rectify, Launch&& launch) {
+  dispatch_tags(dtype, kahan, true, wd, [&](auto dt, auto kh, auto up, auto w) {
     using DT = decltype(dt);
-    constexpr bool K = decltype(kh)::value, U = decltype(up)::value;
+    constexpr bool K = decltype(kh)::value;
     constexpr int W = decltype(w)::value;
-    if (!U) launch(RangerOp<DT, K, U, W, 0, false>{});
-    else if (rectify && la) launch(RangerOp<DT, K, U, W, 0, true>{});
-    else if (rectify) launch(RangerOp<DT, K, U, W, 0, false>{});
-    else if (la) launch(RangerOp<DT, K, U, W, 1, true>{});
-    else launch(RangerOp<DT, K, U, W, 1, false>{});
+    (void)up;
+    if (rectify) launch(RangerOp<DT, K, W, 0>{});
+    else launch(RangerOp<DT, K, W, 1>{});
   });
 }
 
@@ -1637,8 +1636,14 @@ int ranger_list(optimi_group* g, int n_tensors, void* const* param, const void* 
   s.alpha_d = Sd(alpha, dtype);
   s_f32.a = adam_scalars(OPTIMI_F32, step_lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
   s_f32.alpha_d = Sd(alpha, OPTIMI_F32);
-  ranger_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), rectify, la,
-                  [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream, nullptr, &s_f32); });
+  const int wd = adam_wd_mode(weight_decay, flags);
+  if (update && la) {
+    ranger_dispatch(dtype, kahan, wd, rectify, [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream, nullptr, &s_f32); });
+  } else {  // the RAdam step
+    auto launch = [&](auto op) { launch_list<decltype(op)>(g, plan, s.a, stream, nullptr, &s_f32.a); };
+    if (rectify || !update) dispatch<AdamOp, 3>(dtype, kahan, update, wd, launch);
+    else dispatch<RAdamEarlyOp, 3>(dtype, kahan, update, wd, launch);
+  }
   return finish_list(g, plan, stream);
 }
 
@@ -1993,8 +1998,14 @@ int optimi_hip_ranger_single(void* param, const void* grad, void* exp_avg, void*
   RangerScalars s;
   s.a = adam_scalars(dtype, rectify ? lr * rect : lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps);
   s.alpha_d = Sd(alpha, dtype);
-  ranger_dispatch(dtype, kahan, update, adam_wd_mode(weight_decay, flags), rectify, la,
-                  [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
+  const int wd = adam_wd_mode(weight_decay, flags);
+  if (update && la) {
+    ranger_dispatch(dtype, kahan, wd, rectify, [&](auto op) { launch_single<decltype(op)>(e, s, nullptr, stream); });
+  } else {  // the RAdam step
+    auto launch = [&](auto op) { launch_single<decltype(op)>(e, s.a, nullptr, stream); };
+    if (rectify || !update) dispatch<AdamOp, 3>(dtype, kahan, update, wd, launch);
+    else dispatch<RAdamEarlyOp, 3>(dtype, kahan, update, wd, launch);
+  }
   HIP_TRY(hipGetLastError());
   return 0;
 }
