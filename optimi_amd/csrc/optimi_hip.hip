@@ -24,6 +24,7 @@
 
 #include <cmath>
 #include <cstdint>
+#include <cstdio>
 #include <cstdlib>
 #include <atomic>
 #include <cstring>
@@ -1034,19 +1035,25 @@ int finish_list(optimi_group* g, const ListPlan& plan, hipStream_t stream) {
 // count changes), so a workgroup that asks for g granules leaves room for floor(128 / g)
 // workgroups; reachable occupancies are therefore 32, 25, 21, 18, 16, 14, 12, 11, 10, 9, 8, ...
 // The table holds the measured optimum in granules on MI355X with the write-through tile stores
-// (7B-parameter lists; 5 streams = StableAdamW pass 1 and accumulate-only Adam, 6 = pass 2,
-// 7 = Lion / SGD and fp32 Adam, 9 = Adam with Kahan, 11 = Ranger's Lookahead step and Adan without
-// Kahan (22.75 ms at 12 granules against 23.34 at 14, and 23.46 against 23.80), 13 = Adan; entries
-// in between are interpolated).  fp32 Adan (also 11 streams) does best at 17 granules, 7
-// workgroups (a Llama-1B-shaped list: 8.12 ms at 16, 7.98 ms at 17 and 18).  16-bit list launches of fewer than kLongLaunch
-// workgroups (the Llama-1B-shaped list) do best one granule lower, i.e. with one more workgroup
-// resident.  Lists that live in the last-level cache follow the same table (16.8 M parameters:
-// fp32 AdamW 68.9 us at 6 granules, 67.5 us at 10 and 11; bf16 AdamW 48.7 us at 6, 47.0 us at 12;
-// fp32 Adan 131 us at 6, 120 us at 14).  OPTIMI_HIP_WAVES overrides the number of wavefronts
-// per CU for every kernel (nearest reachable count at or above it; 0 = no throttle); read once.
+// (7B-parameter lists):
+//    3 streams  SGD without momentum, accumulate-only Lion and SGD      5 (6.81 TB/s; 6.56 at 4)
+//    4          StableAdamW pass 2 without Kahan                        6 (5 to 7 within 0.5 %)
+//    5, 6       StableAdamW pass 1 and 2, accumulate-only Adam, SGD     8
+//    7          Lion / SGD with Kahan, fp32 Adam                        11
+//    9          Adam with Kahan                                         12
+//    11         Ranger's Lookahead step, Adan without Kahan             12 (22.75 ms; 23.34 ms at 14)
+//    13         Adan with Kahan                                         16
+// and entries in between are interpolated.  fp32 Adan (also 11 streams) does best at 17 granules,
+// 7 workgroups (a Llama-1B-shaped list: 8.12 ms at 16, 7.98 ms at 17 and 18).  16-bit list
+// launches of fewer than kLongLaunch workgroups (the Llama-1B-shaped list) do best one granule
+// lower, i.e. with one more workgroup resident.  Lists that live in the last-level cache follow
+// the same table (16.8 M parameters: fp32 AdamW 68.9 us at 6 granules, 67.5 us at 10 and 11;
+// bf16 AdamW 48.7 us at 6, 47.0 us at 12; fp32 Adan 131 us at 6, 120 us at 14).
+// OPTIMI_HIP_WAVES overrides the number of wavefronts per CU for every kernel (nearest
+// reachable count at or above it; 0 = no throttle); read once.
 constexpr int kLdsGranule = 1280, kLdsGranules = 128;
 constexpr int kMaxStreams = 2 * kMaxArrays;
-constexpr int kBestGranules[kMaxStreams + 1] = {4, 4, 4, 4, 6, 8, 8, 11, 11, 12, 12, 12, 14, 16, 16};
+constexpr int kBestGranules[kMaxStreams + 1] = {5, 5, 5, 5, 6, 8, 8, 11, 11, 12, 12, 12, 14, 16, 16};
 constexpr int64_t kLongLaunch = (int64_t)1 << 22;  // workgroups
 
 int forced_waves() {
@@ -1081,6 +1088,14 @@ LaunchShape launch_shape(int64_t workgroups, bool few) {
   if (!few && !f32 && streams >= 7 && workgroups < kLongLaunch) granules -= 1;
   if (few && (streams == 5 || streams == 6)) granules = 9;
 #ifdef OPTIMI_TUNING
+  {  // raw request for the kernels with this many streams only, tuning builds only
+    char name[32];
+    std::snprintf(name, sizeof(name), "OPTIMI_HIP_LDS_S%d", streams);
+    if (const char* env = std::getenv(name)) {
+      shape.lds = (unsigned)std::strtol(env, nullptr, 10);
+      return shape;
+    }
+  }
   if (const char* env = std::getenv("OPTIMI_HIP_LDS")) {  // raw request, tuning builds only
     shape.lds = (unsigned)std::strtol(env, nullptr, 10);
     return shape;
