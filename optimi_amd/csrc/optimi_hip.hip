@@ -1038,7 +1038,10 @@ int finish_list(optimi_group* g, const ListPlan& plan, hipStream_t stream) {
 // (7B-parameter lists):
 //    3 streams  SGD without momentum, accumulate-only Lion and SGD      5 (6.81 TB/s; 6.56 at 4)
 //    4          StableAdamW pass 2 without Kahan                        6 (5 to 7 within 0.5 %)
-//    5, 6       StableAdamW pass 1 and 2, accumulate-only Adam, SGD     8
+//    5, 6       StableAdamW pass 1 and 2, accumulate-only Adam, SGD     8 (16-bit pass 1, which also reduces and stores a
+//                                                                         partial sum per workgroup: 7 - the 7B list
+//                                                                         in 22.08 ms against 22.44 ms, the 1B list
+//                                                                         in 4.00 ms against 4.07 ms)
 //    7          Lion / SGD with Kahan, fp32 Adam                        11
 //    9          Adam with Kahan                                         12
 //    11         Ranger's Lookahead step, Adan without Kahan             12 (22.75 ms; 23.34 ms at 14)
@@ -1087,6 +1090,7 @@ LaunchShape launch_shape(int64_t workgroups, bool few) {
   if (f32 && streams == 11) granules = 17;
   if (!few && !f32 && streams >= 7 && workgroups < kLongLaunch) granules -= 1;
   if (few && (streams == 5 || streams == 6)) granules = 9;
+  if (!few && !f32 && Op::kReduce) granules = 7;
 #ifdef OPTIMI_TUNING
   {  // raw request for the kernels with this many streams only, tuning builds only
     char name[32];
