@@ -61,7 +61,7 @@ inline int64_t chunks_of(int64_t numel, int64_t chunk) { return (numel + chunk -
 inline int64_t entry_chunk_elems(const TensorEntry& e) { return kChunkBytes / ((e.flags & kEntryF32) ? 4 : 2); }
 
 // Validates a list and writes one entry per tensor.  `lists[a]` may be nullptr for an array the
-// launch does not touch (`need` has its bit clear).  `dtypes`, when not null, gives every
+// launch does not touch (`need` has its bit clear) or that only tensors without elements would use.  `dtypes`, when not null, gives every
 // tensor's own dtype (a mixed list); otherwise all tensors have `dtype`.  Arrays in
 // `low_precision_only` (the Kahan buffer) exist for 16-bit tensors only: an fp32 tensor's
 // pointer there is ignored.  `max_chunks` bounds the launch (the grid is chunks x workgroups
@@ -73,8 +73,6 @@ inline int build_entries(int n_tensors, const void* const* const* lists, int n_a
   if (!dtypes && !valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
   if (n_arrays < 0 || n_arrays > kMaxArrays) return OPTIMI_ERR_SIZE;
   if (n_tensors > 0 && (!numel || !out)) return OPTIMI_ERR_NULL;
-  for (int a = 0; a < n_arrays; ++a)
-    if ((need & bit(a)) && n_tensors > 0 && (!lists || !lists[a])) return OPTIMI_ERR_NULL;
   int64_t n_chunks = 0;
   for (int t = 0; t < n_tensors; ++t) {
     const int dt = dtypes ? dtypes[t] : dtype;
@@ -91,7 +89,7 @@ inline int build_entries(int n_tensors, const void* const* const* lists, int n_a
     for (int a = 0; a < n_arrays; ++a) {
       if (!(need & bit(a))) continue;
       if (dt == OPTIMI_F32 && (low_precision_only & bit(a))) continue;
-      const void* p = lists[a][t];
+      const void* p = (lists && lists[a]) ? lists[a][t] : nullptr;  // a missing list is a list of null pointers
       if (!p && numel[t] > 0) return OPTIMI_ERR_NULL;
       const uintptr_t u = (uintptr_t)p;
       if (u % eb) return OPTIMI_ERR_ALIGN;

@@ -956,6 +956,7 @@ class ReleaseHookCore {
       const at::Tensor& p0 = items[first].p;
       at::ScalarType low = at::kFloat;
       std::vector<void*> ptr[kMaxTensors];
+      std::vector<char> has[kMaxTensors];  // the array exists for the tensor (a tensor without elements has no address)
       std::vector<int64_t> numel;
       std::vector<int> dtypes;
       for (size_t i = first; i < items.size(); ++i) {
@@ -967,7 +968,10 @@ class ReleaseHookCore {
         }
         done[i] = 1;
         const StepCall c = pack(*items[i].e, h, p, items[i].g, momentum);
-        for (int a = 0; a < nt; ++a) ptr[a].push_back(c.t[a].has_value() ? c.t[a]->data_ptr() : nullptr);
+        for (int a = 0; a < nt; ++a) {
+          ptr[a].push_back(c.t[a].has_value() ? c.t[a]->data_ptr() : nullptr);
+          has[a].push_back(c.t[a].has_value());
+        }
         if (p.scalar_type() == at::kFloat) ptr[nt - 1].back() = nullptr;  // no Kahan buffer for fp32
         numel.push_back(p.numel());
         dtypes.push_back(dtype_code(p));
@@ -977,7 +981,7 @@ class ReleaseHookCore {
         int present = -1;
         for (size_t i = 0; i < ptr[a].size(); ++i) {
           if (a == nt - 1 && dtypes[i] == OPTIMI_F32) continue;
-          const int here = ptr[a][i] != nullptr;
+          const int here = has[a][i];
           TORCH_CHECK(present < 0 || present == here, "optimi_amd: a state buffer is missing for some parameters of a group");
           present = here;
         }

@@ -170,6 +170,9 @@ static void check_rejections() {
   const void* const* holes[2] = {a, nullptr};
   CHECK(build_entries(2, holes, 2, 3, numel, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_ERR_NULL, "missing needed list");
   CHECK(build_entries(2, holes, 2, 1, numel, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_OK, "an unneeded list may be null");
+  int64_t both_empty[2] = {0, 0};
+  CHECK(build_entries(2, holes, 2, 3, both_empty, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_OK && n == 0,
+        "a needed list may be null when no tensor has elements");
   const void* b[2] = {(const void*)0x1000, nullptr};
   const void* const* with_null[2] = {a, b};
   CHECK(build_entries(2, with_null, 2, 3, numel, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_ERR_NULL, "null buffer of a non-empty tensor");

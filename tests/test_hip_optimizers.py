@@ -550,3 +550,47 @@ def test_mixed_group_with_state_dict_roundtrip(case, hip_device):
             fresh.load_state_dict(torch.load(blob, weights_only=True))
             opt = fresh
     assert opt.state[params[0]]["exp_avg"].dtype == torch.bfloat16 and opt.state[params[1]]["exp_avg"].dtype == torch.float32
+
+
+@pytest.mark.parametrize("release", [False, True], ids=["step", "gradient_release"])
+def test_zero_dim_and_empty_parameters(release, hip_device):
+    """A 0-dim parameter (a learnable temperature) and a parameter without elements beside ordinary
+    ones: both calling forms accept them, the former is stepped, the latter is left alone."""
+    gen = torch.Generator().manual_seed(12)
+    shapes = [(), (0, 7), (50, 3), (0,)]
+    params = [torch.nn.Parameter((torch.randn(s, generator=gen) * 0.5).to(hip_device)) for s in shapes]
+    hyper = dict(lr=1e-2, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
+    opt = optimi_amd.AdamW(params, gradient_release=release, **hyper)
+    ref = ForLoopRun("adamw", [p.detach().cpu().clone() for p in params], gradient_release=release, **hyper)
+    hook = opt._native_hook() if release else None
+    for _ in range(4):
+        grads = [(torch.randn(s, generator=gen) * 1e-2) for s in shapes]
+        if release:
+            for i in reversed(range(len(params))):
+                params[i].grad = grads[i].to(hip_device)
+                hook(params[i])
+                ref.step_param(i, grads[i].clone())
+        else:
+            for p, g in zip(params, grads):
+                p.grad = g.to(hip_device)
+            opt.step()
+            opt.zero_grad()
+            ref.step([g.clone() for g in grads])
+    opt.step()  # under gradient release: launches whatever is still parked
+    torch.cuda.synchronize()
+    for i, (p, q) in enumerate(zip(params, ref.params)):
+        assert p.shape == q.shape
+        if p.numel():
+            G.assert_close_to_reference(p, q, f"param {i} of shape {tuple(p.shape)}", is_param=True)
+    # a group that holds nothing but empty low-precision parameters (Kahan buffers without an address)
+    hollow = [torch.nn.Parameter(torch.zeros(s, dtype=torch.bfloat16, device=hip_device)) for s in [(0, 4), (0,)]]
+    opt = optimi_amd.AdamW(hollow, gradient_release=release, **hyper)
+    hook = opt._native_hook() if release else None
+    for _ in range(3):
+        for p in hollow:
+            p.grad = torch.zeros_like(p)
+            if release:
+                hook(p)
+        opt.step()
+        opt.zero_grad()
+    torch.cuda.synchronize()
