@@ -594,3 +594,34 @@ def test_zero_dim_and_empty_parameters(release, hip_device):
         opt.step()
         opt.zero_grad()
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("n_params", [6, 24], ids=["kernel_argument_table", "device_tables"])
+@pytest.mark.parametrize("case", ["adamw", "stableadamw", "adan"])
+def test_changing_subset_of_gradients_and_a_moving_learning_rate(case, n_params, hip_device):
+    """Steps on which only some parameters have a gradient (frozen branches, unused heads) and a
+    learning rate a scheduler moves every step: the launch list changes from step to step, the
+    group's one step counter still advances for everyone (optimi/adam.py:164-182), and parameters
+    without a gradient keep their values and states."""
+    cls, oname, hyper = CASES[case]
+    gen = torch.Generator().manual_seed(21)
+    shapes = [[(40, 30), (8200,), (64,), (3, 5, 7)][i % 4] for i in range(n_params)]
+    params = [torch.nn.Parameter((torch.randn(s, generator=gen) * 0.02).to(torch.bfloat16).to(hip_device)) for s in shapes]
+    opt = cls(params, **hyper)
+    ref = oracle_for(oname, params, hyper)
+    sched = torch.optim.lr_scheduler.LambdaLR(opt, lambda step: 1.0 / (1.0 + 0.25 * step))
+    base_lr = hyper["lr"]
+    for it in range(8):
+        present = [(i + it) % 3 != 0 for i in range(n_params)]  # two thirds of the parameters; a third is first seen on the second step
+        grads = []
+        for p, on in zip(params, present):
+            p.grad = (torch.randn(p.shape, generator=gen) * 1e-3).to(p.dtype).to(hip_device) if on else None
+            grads.append(p.grad.detach().cpu().clone() if on else None)
+        ref.hyper["lr"] = base_lr / (1.0 + 0.25 * it)
+        if ref.hyper.get("decouple_lr"):
+            ref.hyper["max_lr"] = base_lr
+        opt.step()
+        sched.step()
+        opt.zero_grad()
+        ref.step(grads)
+    compare(opt, params, ref, f"{case} changing subsets")
