@@ -625,3 +625,42 @@ def test_changing_subset_of_gradients_and_a_moving_learning_rate(case, n_params,
         opt.zero_grad()
         ref.step(grads)
     compare(opt, params, ref, f"{case} changing subsets")
+
+
+@pytest.mark.parametrize("case", ["adamw", "stableadamw", "ranger"])
+def test_deepcopy_continues_like_the_original(case, hip_device):
+    """``copy.deepcopy`` of an optimizer (what EMA and checkpointing helpers do) copies parameters
+    and states and must leave the launch workspaces behind: original and copy then step their own
+    parameters to the same bits."""
+    import copy
+
+    cls, _, hyper = CASES[case]
+    gen = torch.Generator().manual_seed(31)
+    shapes = [(40, 30), (8200,), (64,)] * 7  # 21 tensors: device tables
+    params = [torch.nn.Parameter((torch.randn(s, generator=gen) * 0.02).to(torch.bfloat16).to(hip_device)) for s in shapes]
+    opt = cls(params, **hyper)
+
+    def run(optimizer, grads):
+        for p, g in zip(optimizer.param_groups[0]["params"], grads):
+            p.grad = g.clone()
+        optimizer.step()
+        optimizer.zero_grad()
+
+    def draw():
+        return [(torch.randn(s, generator=gen) * 1e-3).to(torch.bfloat16).to(hip_device) for s in shapes]
+
+    for _ in range(3):
+        run(opt, draw())
+    twin = copy.deepcopy(opt)
+    twin_params = twin.param_groups[0]["params"]
+    assert all(a is not b and a.data_ptr() != b.data_ptr() for a, b in zip(params, twin_params))
+    for _ in range(4):
+        grads = draw()
+        run(opt, grads)
+        run(twin, grads)
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(zip(params, twin_params)):
+        G.assert_bits_equal(a, b, f"{case} param {i}")
+        for key in G.STATE_KEYS:
+            if key in opt.state[a] and torch.is_tensor(opt.state[a][key]) and opt.state[a][key].numel() == a.numel():
+                G.assert_bits_equal(opt.state[a][key], twin.state[b][key], f"{case} {key} {i}")
