@@ -664,3 +664,28 @@ def test_deepcopy_continues_like_the_original(case, hip_device):
         for key in G.STATE_KEYS:
             if key in opt.state[a] and torch.is_tensor(opt.state[a][key]) and opt.state[a][key].numel() == a.numel():
                 G.assert_bits_equal(opt.state[a][key], twin.state[b][key], f"{case} {key} {i}")
+
+
+def test_step_with_a_closure(hip_device):
+    """``step(closure)`` re-evaluates the model with gradients enabled, steps on the gradients the
+    closure produced and returns its loss (optimi/adam.py:152-155)."""
+    model, params = make(torch.bfloat16, hip_device, seed=5)
+    opt = optimi_amd.AdamW(params, lr=1e-3)
+    ref = oracle_for("adamw", params, dict(lr=1e-3))
+    gen = torch.Generator().manual_seed(2)
+    x = torch.randn(16, 128, generator=gen).to(torch.bfloat16).to(hip_device)
+    y = torch.randn(16, 1, generator=gen).to(torch.bfloat16).to(hip_device)
+    calls = []
+
+    def closure():
+        opt.zero_grad()
+        loss = torch.nn.functional.mse_loss(model(x), y)
+        loss.backward()
+        calls.append(torch.is_grad_enabled())
+        return loss
+
+    for _ in range(3):
+        loss = opt.step(closure)
+        assert loss is not None and loss.requires_grad and calls[-1] is True
+        ref.step([p.grad.detach().cpu().clone() for p in params])
+    compare(opt, params, ref, "closure")
