@@ -689,3 +689,37 @@ def test_step_with_a_closure(hip_device):
         assert loss is not None and loss.requires_grad and calls[-1] is True
         ref.step([p.grad.detach().cpu().clone() for p in params])
     compare(opt, params, ref, "closure")
+
+
+@pytest.mark.parametrize("case", ["adamw", "stableadamw", "lion"])
+def test_parameters_that_are_views_into_a_flat_buffer(case, hip_device):
+    """Parameters carved out of one flat buffer (flattened-parameter wrappers do this) start wherever
+    the previous one ended, so most are not 16-byte aligned while their freshly allocated states and
+    gradients are: the kernels take the element-wise path for such a tensor and must not touch its
+    neighbours in the buffer."""
+    cls, oname, hyper = CASES[case]
+    gen = torch.Generator().manual_seed(41)
+    sizes = [1001, 8195, 3, 4099, 70000]
+    for dtype in (torch.bfloat16, torch.float32):
+        flat = torch.full((sum(sizes) + 2 * len(sizes) + 9,), 7.0, dtype=dtype, device=hip_device)
+        params, spans, at = [], [], 1  # one element in: even the first view is off the 16-byte grid
+        for n in sizes:
+            view = flat[at:at + n]
+            view.copy_((torch.randn(n, generator=gen) * 0.02).to(dtype))
+            params.append(torch.nn.Parameter(view))
+            spans.append((at, at + n))
+            at += n + 2  # two untouched elements between neighbours
+        assert any(p.data_ptr() % 16 for p in params)
+        opt = cls(params, **hyper)
+        ref = oracle_for(oname, params, hyper)
+        for _ in range(4):
+            for p in params:
+                p.grad = (torch.randn(p.shape, generator=gen) * 1e-3).to(dtype).to(hip_device)
+            ref.step([p.grad.detach().cpu().clone() for p in params])
+            opt.step()
+            opt.zero_grad()
+        compare(opt, params, ref, f"{case} {dtype} views")
+        keep = torch.ones_like(flat, dtype=torch.bool)
+        for a, b in spans:
+            keep[a:b] = False
+        assert bool((flat[keep] == 7.0).all()), "wrote between the views"
