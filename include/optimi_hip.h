@@ -21,8 +21,9 @@
  *     the call returns without waiting for it.
  *   - `kahan_comp` may be NULL whenever the Kahan branch is not taken (fp32 tensors,
  *     OPTIMI_KAHAN unset, or OPTIMI_UPDATE unset).  "Low precision" below means bf16 or fp16.
- *   - buffers aligned to 16 bytes take the vectorised path; any other alignment is
- *     accepted and runs an element-wise path.
+ *   - buffers need only be aligned to their element size.  Tensors whose buffers are all
+ *     16-byte aligned take the streaming path; others run the same 16-byte vectors through
+ *     element-aligned accesses (about 10 % slower).
  */
 #ifndef OPTIMI_HIP_H
 #define OPTIMI_HIP_H

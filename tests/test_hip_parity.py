@@ -147,7 +147,7 @@ def test_random_lists_match_both_oracles(cfg, dtype, kahan, hip_device):
 
 @pytest.mark.parametrize("cfg", ["adamw", "lion", "stableadamw", "adan", "sgd_momentum", "radam", "ranger"])
 def test_unaligned_buffers(cfg, hip_device):
-    """Views that start 2 bytes (bf16) past a 16-byte boundary take the element-wise path."""
+    """Views that start 2 bytes (bf16) past a 16-byte boundary take the element-aligned vector path."""
     hyper, name = CONFIGS[cfg], OPT_OF[cfg]
     sizes = [5, 600, 9000]
     params, grads = draw(sizes, torch.bfloat16, 4, seed=5)
