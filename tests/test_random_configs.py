@@ -6,6 +6,8 @@ stepping with accumulate-only micro-steps.
 * CPU: the C emulator against the torch for-loop restatement (each pinned by the reference's
   fixtures on the configurations those cover; here they pin each other elsewhere).
 * GPU: the HIP kernels, through the C ABI, against the C emulator.
+* Misaligned views (GPU): every other configuration again with parameters and gradients one or two
+  elements off the 16-byte grid and sizes that are not multiples of the vector, against the emulator.
 * Mixed lists: the same configurations with every other tensor in fp32 beside the 16-bit ones,
   one launch on the GPU (the ``_multi_mixed`` entry points).
 
@@ -142,3 +144,31 @@ def test_hip_matches_emulator(seed, hip_device):
     sca = ScalarRun(name, [p.clone() for p in params], gradient_release=release, **mode, **hyper)
     drive([(hip, lambda g: g.to(hip_device)), (sca, torch.clone)], grads, release)
     G.compare_engines(hip, sca, f"seed {seed}: {name} {dtype} {hyper} release={release}", exact=name != "stableadamw")
+
+
+ODD_SIZES = [33, 97, 515, 4129, 8200, 7]
+
+
+def _off_grid(t, k, device):
+    """``t`` on ``device`` as a view that starts ``k`` elements into its buffer."""
+    buf = torch.zeros(t.numel() + 16, dtype=t.dtype, device=device)
+    view = buf[k:k + t.numel()].view(t.shape)
+    view.copy_(t)
+    return view
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(0, N_CONFIGS, 2))
+def test_hip_matches_emulator_on_misaligned_views(seed, hip_device):
+    from hip_engine import HipRun
+
+    name, dtype, hyper, release, data_seed = draw_config(seed)
+    gen = torch.Generator().manual_seed(data_seed)
+    params = [(torch.randn(n, generator=gen) * 0.02).to(dtype) for n in ODD_SIZES]
+    grads = [[(torch.randn(n, generator=gen) * 1e-3 * (1.0, 4.0, 0.25)[t % 3]).to(dtype) for n in ODD_SIZES] for t in range(5)]
+    mode = engine_mode(name, hyper)
+    hip = HipRun(name, [_off_grid(p, (i + seed) % 3, hip_device) for i, p in enumerate(params)], gradient_release=release,
+                 **mode, **hyper)
+    sca = ScalarRun(name, [p.clone() for p in params], gradient_release=release, **mode, **hyper)
+    drive([(hip, lambda g: _off_grid(g, (seed // 2) % 2 + 1, hip_device)), (sca, torch.clone)], grads, release)
+    G.compare_engines(hip, sca, f"seed {seed}: {name} {dtype} {hyper} release={release}, misaligned", exact=name != "stableadamw")
