@@ -85,19 +85,21 @@ __device__ __forceinline__ void store16(void* base, int64_t byte_off, u32x4 v) {
   __builtin_nontemporal_store(v, (OPTIMI_GLOBAL u32x4*)((uintptr_t)base + (uintptr_t)byte_off));
 }
 // The same vector at an address that is only aligned to one element (ELEM = 2 or 4 bytes): the
-// packed type tells the compiler so, and it emits what the target guarantees to work (one
-// 16-byte access on gfx950, whose memory unit handles unaligned global accesses).
-template <int ELEM>
-struct __attribute__((packed, aligned(ELEM))) UnalignedVec {
-  u32x4 v;
-};
+// reduced alignment of the type tells the compiler so, and it emits what the target guarantees
+// to work (one 16-byte access on gfx950, whose memory unit handles unaligned global accesses).
+typedef u32x4 u32x4_align2 __attribute__((aligned(2)));
+typedef u32x4 u32x4_align4 __attribute__((aligned(4)));
 template <int ELEM>
 __device__ __forceinline__ u32x4 load16_unaligned(const void* base, int64_t byte_off) {
-  return ((const OPTIMI_GLOBAL UnalignedVec<ELEM>*)((uintptr_t)base + (uintptr_t)byte_off))->v;
+  const uintptr_t at = (uintptr_t)base + (uintptr_t)byte_off;
+  if (ELEM == 2) return __builtin_nontemporal_load((const OPTIMI_GLOBAL u32x4_align2*)at);
+  return __builtin_nontemporal_load((const OPTIMI_GLOBAL u32x4_align4*)at);
 }
 template <int ELEM>
 __device__ __forceinline__ void store16_unaligned(void* base, int64_t byte_off, u32x4 v) {
-  ((OPTIMI_GLOBAL UnalignedVec<ELEM>*)((uintptr_t)base + (uintptr_t)byte_off))->v = v;
+  const uintptr_t at = (uintptr_t)base + (uintptr_t)byte_off;
+  if (ELEM == 2) __builtin_nontemporal_store(v, (OPTIMI_GLOBAL u32x4_align2*)at);
+  else __builtin_nontemporal_store(v, (OPTIMI_GLOBAL u32x4_align4*)at);
 }
 
 // The store of a full tile: a buffer store with the sc0 sc1 cache policy, i.e. written through
