@@ -114,7 +114,9 @@ def numel(shape):
     return n
 
 
-def make_tensors(shapes, dtype, device, seed, std, ones_for_1d=False):
+def make_tensors(shapes, dtype, device, seed, std, ones_for_1d=False, misalign=0):
+    """``misalign`` = k > 0: every tensor is a view that starts k elements into its own buffer, i.e. off
+    the 16-byte grid (what a view into a flat buffer or a gradient inside a bucket looks like)."""
     import torch
 
     gen = torch.Generator(device=device).manual_seed(seed)
@@ -122,11 +124,17 @@ def make_tensors(shapes, dtype, device, seed, std, ones_for_1d=False):
     out = []
     for s, dt in zip(shapes, dtypes):
         if ones_for_1d and len(s) == 1:
-            out.append(torch.ones(s, dtype=dt, device=device))
+            t = torch.ones(s, dtype=dt, device=device)
         else:
-            t = torch.empty(s, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
-            out.append(t.to(dt))
-            del t
+            f = torch.empty(s, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
+            t = f.to(dt)
+            del f
+        if misalign:
+            buf = torch.empty(t.numel() + 16, dtype=dt, device=device)
+            view = buf[misalign:misalign + t.numel()].view(s)
+            view.copy_(t)
+            t = view
+        out.append(t)
     return out
 
 
@@ -286,8 +294,9 @@ def list_bench(workload, args, steps, warmup):
     if is_fp32:  # the average over the list: 28 bytes per fp32 parameter (four arrays read, three written)
         bytes_per_param = (bytes_per_param * (n_params - n_fp32) + 28 * n_fp32) / n_params
 
-    params = [torch.nn.Parameter(p) for p in make_tensors(shapes, dtypes, device, 0, 0.02, ones_for_1d=True)]
-    grad_sets = [make_tensors(shapes, dtypes, device, 100 + i, 1e-3) for i in range(max(1, args.grad_sets))]
+    misalign = getattr(args, "misalign", 0)
+    params = [torch.nn.Parameter(p) for p in make_tensors(shapes, dtypes, device, 0, 0.02, ones_for_1d=True, misalign=misalign)]
+    grad_sets = [make_tensors(shapes, dtypes, device, 100 + i, 1e-3, misalign=misalign) for i in range(max(1, args.grad_sets))]
     opt = getattr(optimi_amd, cls_name)(params, **kwargs)
 
     def one_step(i):
@@ -351,7 +360,7 @@ def list_bench(workload, args, steps, warmup):
         "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype],
         "data": "synthetic",
         "config": {"workload": workload, "optimizer": cls_name, "n_tensors": len(shapes), "n_params": n_params,
-                   **({"n_params_fp32": n_fp32} if is_fp32 else {}),
+                   **({"n_params_fp32": n_fp32} if is_fp32 else {}), **({"misalign_elements": misalign} if misalign else {}),
                    "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()},
                    "grad_sets": len(grad_sets)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -398,6 +407,9 @@ def main():
     ap.add_argument("--grad-sets", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="measure the named workload only, not the other configurations")
+    ap.add_argument("--misalign", type=int, default=0,
+                    help="list workloads: make every parameter and gradient a view that starts this many elements into "
+                         "its buffer (off the 16-byte grid); the optimizer states stay aligned")
     ap.add_argument("--no-coalesce", action="store_true",
                     help="gradient-release workloads: launch every tensor from its own hook instead of parking small ones")
     ap.add_argument("--copy-probe-bytes", type=int, default=0,
