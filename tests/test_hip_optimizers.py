@@ -723,3 +723,69 @@ def test_parameters_that_are_views_into_a_flat_buffer(case, hip_device):
         for a, b in spans:
             keep[a:b] = False
         assert bool((flat[keep] == 7.0).all()), "wrote between the views"
+
+
+@pytest.mark.parametrize("case", ["adamw", "stableadamw", "adan"])
+def test_dense_parameter_with_permuted_strides(case, hip_device):
+    """A parameter that is dense in memory but not contiguous (a transposed weight, a
+    channels-last filter): its states are created with the same strides (``zeros_like`` with
+    ``preserve_format``), its gradient is brought to them, and the step is element-wise, so the
+    result equals the oracle's on the logical tensor."""
+    cls, oname, hyper = CASES[case]
+    gen = torch.Generator().manual_seed(23)
+    for dtype in (torch.bfloat16, torch.float32):
+        w = torch.nn.Parameter((torch.randn(96, 130, generator=gen) * 0.02).to(dtype).to(hip_device).t())
+        f = torch.nn.Parameter((torch.randn(6, 5, 7, 3, generator=gen) * 0.02).to(dtype).to(hip_device)
+                               .contiguous(memory_format=torch.channels_last))
+        assert not w.is_contiguous() and not f.is_contiguous()
+        params = [w, f]
+        opt = cls(params, **hyper)
+        ref = oracle_for(oname, params, hyper)
+        for step in range(4):
+            for p in params:
+                g = (torch.randn(p.shape, generator=gen) * 1e-3).to(dtype).to(hip_device)  # contiguous: other strides than p
+                p.grad = g if step % 2 else torch.empty_like(p).copy_(g)  # on even steps already in p's layout
+            ref.step([p.grad.detach().cpu().contiguous() for p in params])
+            opt.step()
+            opt.zero_grad()
+        assert opt.state[w]["exp_avg"].stride() == w.stride() and opt.state[f]["exp_avg"].stride() == f.stride()
+        compare(opt, params, ref, f"{case} {dtype} permuted")
+
+
+def test_two_optimizers_stepping_from_two_threads(hip_device):
+    """Two optimizers, each driven by its own Python thread on its own stream: every launch uses
+    the calling thread's current stream and the optimizer's own launch workspace, so the threads
+    do not disturb each other (20 tensors each: device tables; StableAdamW: reduction scratch)."""
+    import threading
+
+    shapes = [(300, 70), (8200,), (5,), (4096, 16), (513,)] * 4
+    results, errors = {}, []
+
+    def work(name, seed):
+        try:
+            cls, oname, hyper = CASES[name]
+            gen = torch.Generator().manual_seed(seed)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                params = [torch.nn.Parameter((torch.randn(s, generator=gen) * 0.02).bfloat16().to(hip_device)) for s in shapes]
+                opt = cls(params, **hyper)
+                ref = oracle_for(oname, params, hyper)
+                for _ in range(6):
+                    grads = [(torch.randn(s, generator=gen) * 1e-3).bfloat16() for s in shapes]
+                    for p, g in zip(params, grads):
+                        p.grad = g.to(hip_device)
+                    opt.step()
+                    ref.step(grads)
+                stream.synchronize()
+            results[name] = (opt, params, ref)
+        except Exception as exc:  # noqa: BLE001 - reported by the main thread
+            errors.append((name, exc))
+
+    threads = [threading.Thread(target=work, args=(n, i)) for i, n in enumerate(["adamw", "stableadamw"])]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for name, (opt, params, ref) in results.items():
+        compare(opt, params, ref, f"threaded {name}")
