@@ -182,6 +182,119 @@ def cpu_baseline(cls_name, kwargs, dtype, shapes, budget_s=25.0):
     }
 
 
+# What one step of each optimizer reads and writes, pass by pass: (arrays written in place, arrays only read).
+# "p" is the parameter, "g" the gradient, the rest are state keys; the Kahan buffer exists for 16-bit tensors only.
+ACCESS_MIX = {
+    "AdamW": [(("p", "exp_avg", "exp_avg_sq", "kahan_comp"), ("g",))],
+    "RAdam": [(("p", "exp_avg", "exp_avg_sq", "kahan_comp"), ("g",))],
+    "Ranger": [(("p", "exp_avg", "exp_avg_sq", "kahan_comp"), ("g",))],
+    "Lion": [(("p", "exp_avg", "kahan_comp"), ("g",))],
+    "SGD": [(("p", "exp_avg", "kahan_comp"), ("g",))],
+    "StableAdamW": [(("exp_avg", "exp_avg_sq"), ("g",)), (("p", "kahan_comp"), ("exp_avg", "exp_avg_sq"))],
+    "Adan": [(("p", "exp_avg", "exp_avg_diff", "exp_avg_sq", "prev_grad", "kahan_comp"), ("g",))],
+}
+
+
+def mix_ceiling(cls_name, opt, params, grads, reps=5, granules=0):
+    """The ceiling of a workload's access mix, measured on the workload's own tensors: the library's
+    traffic probe (optimi_hip_stream_probe: the step's launch - same kernel, tiles, loads, stores, tables,
+    throttle - with no arithmetic) over the arrays one step reads and writes.  A list that holds fp32 and
+    16-bit tensors takes one probe launch per dtype.  Returns the mean seconds per step-equivalent.  The
+    tensors hold meaningless bits afterwards, so this runs when the workload is done with them."""
+    import torch
+
+    from optimi_amd import cabi
+
+    L = cabi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    launches = []  # (group, n, table, keep-alive, bytes, n_read, n_write)
+    for written, read_only in ACCESS_MIX[cls_name]:
+        for low in (True, False):
+            idx = [i for i, p in enumerate(params) if (p.dtype != torch.float32) == low]
+            if not idx:
+                continue
+
+            def array(key, i):
+                if key == "p":
+                    return params[i].data
+                if key == "g":
+                    return grads[i]
+                return opt.state[params[i]][key]
+
+            keys = [k for k in written + read_only if low or k != "kahan_comp"]
+            n_write = len([k for k in written if low or k != "kahan_comp"])
+            cols = [[array(k, i).data_ptr() for i in idx] for k in keys]
+            for k in keys:
+                assert all(array(k, i).numel() == params[i].numel() for i in idx), k
+            table, keep = cabi.ptr_table(cols)
+            sizes = cabi.i64_array(params[i].numel() * params[i].element_size() for i in idx)
+            launches.append((cabi.Group(), len(idx), table, keep, sizes, len(keys), n_write))
+
+    def once():
+        for grp, n, table, _, sizes, n_read, n_write in launches:
+            cabi.check(L.optimi_hip_stream_probe(grp.handle, n, table, sizes, n_read, n_write, granules, 0, stream),
+                       "optimi_hip_stream_probe")
+
+    for _ in range(2):
+        once()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        once()
+    stop.record()
+    torch.cuda.synchronize()
+    seconds = start.elapsed_time(stop) * 1e-3 / reps
+    for grp, *_ in launches:
+        grp.close()
+    return seconds, "+".join(f"{r}r/{w}w" for _, _, _, _, _, r, w in launches)
+
+
+def probe_sweep(args):
+    """The library's traffic probe over the Llama-7B-shaped list (290 tensors, 13.5 GB per array, bf16
+    values as the optimizers see them) for the access mixes of the optimizers, at the occupancy the
+    library picks for each and at every occupancy around it: one JSON line, GB/s per (mix, granules).
+    A workgroup that asks for g LDS granules leaves room for floor(128 / g) workgroups on a CU."""
+    import torch
+
+    from optimi_amd import cabi
+
+    device = torch.device("cuda:0")
+    shapes = llama_shapes(4096, 11008, 32)
+    n_params = sum(numel(s) for s in shapes)
+    arrays = [make_tensors(shapes, torch.bfloat16, device, 40 + a, 0.02 if a == 0 else 1e-3) for a in range(7)]
+    L = cabi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    sizes = cabi.i64_array(numel(s) * 2 for s in shapes)
+    grp = cabi.Group()
+    mixes = [(2, 1), (3, 2), (4, 2), (4, 3), (5, 4), (6, 5), (7, 6)]
+    sweep = [0, 5, 6, 7, 8, 9, 10, 11, 12, 14, 16, 18, 21]
+    table_out = {}
+    for n_read, n_write in mixes:
+        table, keep = cabi.ptr_table([[t.data_ptr() for t in arrays[a]] for a in range(n_read)])
+        row = {}
+        for granules in sweep:
+            def once():
+                cabi.check(L.optimi_hip_stream_probe(grp.handle, len(shapes), table, sizes, n_read, n_write, granules, 0, stream),
+                           "optimi_hip_stream_probe")
+            for _ in range(2):
+                once()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            start.record()
+            for _ in range(args.steps):
+                once()
+            stop.record()
+            torch.cuda.synchronize()
+            ms = start.elapsed_time(stop) / args.steps
+            row["library" if granules == 0 else str(granules)] = round((n_read + n_write) * 2 * n_params / ms / 1e6, 1)
+        table_out[f"{n_read}r/{n_write}w"] = row
+        del keep
+    grp.close()
+    print(json.dumps({"probe_sweep": table_out, "unit": "GB/s", "columns": "LDS granules per workgroup (library = the library's own choice)",
+                      "list": "llama7b", "n_tensors": len(shapes), "bytes_per_array": 2 * n_params, "steps": args.steps}), flush=True)
+
+
 def stress_shapes(n_tensors=10_000, lo=128, hi=65536, seed=6):
     """Sizes log-uniform in [lo, hi]: the many-small-tensors list of the gradient-release stress case."""
     import math
@@ -375,6 +488,12 @@ def list_bench(workload, args, steps, warmup):
     }
     if traffic is None:
         out["roofline"]["traffic_note"] = "no hardware-counter profile is kept for this workload"
+    if not args.no_probe_mix:
+        # same bytes, same tensors, same launch, no arithmetic: what this access mix can reach here
+        seconds, mix = mix_ceiling(cls_name, opt, params, grad_sets[0])
+        ceiling = algo_bytes / seconds / 1e9
+        out["roofline"].update(mix_ceiling_gbps=ceiling, mix_ceiling_frac=ceiling / HBM_PEAK_GBPS, mix=mix,
+                               frac_of_mix_ceiling=achieved / ceiling)
     del opt, params, grad_sets
     # the CPU baseline is timed for lists of one dtype only
     return out, (None if is_fp32 else (cls_name, kwargs, dtype, shapes))
@@ -393,6 +512,8 @@ def brief(line):
            "unit": line["unit"], "value": line["value"]}
     if "kernel_ms" in r:
         out.update(kernel_ms=r["kernel_ms"], kernel_ms_min=r["kernel_ms_min"], bytes_per_param=r["bytes_per_param"])
+        if "mix_ceiling_gbps" in r:
+            out.update(mix_ceiling_gbps=r["mix_ceiling_gbps"], mix=r["mix"], frac_of_mix_ceiling=r["frac_of_mix_ceiling"])
     else:
         out.update(timed="wall clock over backward passes", empty_hook_pass_ms=line["config"]["empty_hook_pass_ms"])
     return out
@@ -410,6 +531,12 @@ def main():
     ap.add_argument("--misalign", type=int, default=0,
                     help="list workloads: make every parameter and gradient a view that starts this many elements into "
                          "its buffer (off the 16-byte grid); the optimizer states stay aligned")
+    ap.add_argument("--no-probe-mix", action="store_true",
+                    help="list workloads: do not measure the ceiling of the workload's access mix with the library's "
+                         "traffic probe after the timed steps")
+    ap.add_argument("--probe-sweep", action="store_true",
+                    help="instead of a workload: the traffic probe over the Llama-7B-shaped list for every optimizer's "
+                         "access mix, at the library's occupancy and at every occupancy around it (--steps launches each)")
     ap.add_argument("--no-coalesce", action="store_true",
                     help="gradient-release workloads: launch every tensor from its own hook instead of parking small ones")
     ap.add_argument("--copy-probe-bytes", type=int, default=0,
@@ -443,6 +570,10 @@ def main():
                        "optimi_hip_copy_probe")
         torch.cuda.synchronize()
         del src, dst
+
+    if args.probe_sweep:
+        probe_sweep(args)
+        return
 
     # Between workloads the freed tensors stay in torch's caching allocator and are handed out again
     # (the 7B-shaped workloads share their shapes).  Returning them to the driver and allocating

@@ -49,11 +49,13 @@ enum optimi_flags {
   OPTIMI_RECTIFY = 64,    /* RAdam/Ranger: rho > 5, take the rectified Adam step (optimi/radam.py:269-277) */
   OPTIMI_LOOKAHEAD = 128, /* Ranger: this step synchronises with the slow weights, step % k == 0
                              (optimi/ranger.py:452, 471)                                           */
-  OPTIMI_COLD = 256       /* whole-list entry points: the tensors were not touched recently (they are a
+  OPTIMI_COLD = 256,      /* whole-list entry points: the tensors were not touched recently (they are a
                              slice of a larger model, e.g. small tensors gathered during gradient
                              release).  A hint: a short list otherwise counts as resident in the
                              last-level cache and is read with cached instead of streaming loads.
                              Results do not depend on it.  No counterpart in the reference.        */
+  OPTIMI_PROBE_SCRAMBLE = 512 /* optimi_hip_stream_probe only: the written arrays get new bits (a mix of
+                             everything that was read) instead of keeping theirs                    */
 };
 
 enum optimi_status {
@@ -273,6 +275,26 @@ int optimi_hip_ranger_single(void* param, const void* grad, void* exp_avg, void*
  * the practical bandwidth ceiling and to scale hardware byte counters.
  * ------------------------------------------------------------------------------- */
 int optimi_hip_copy_probe(void* dst, const void* src, int64_t bytes, optimi_stream_t stream);
+
+/* Measurement aid (no counterpart in the reference; nothing of the optimizers calls it): the
+ * memory traffic of a step without its arithmetic.  Array a of tensor i is arrays[a][i], bytes[i]
+ * bytes long (a multiple of 16, every pointer 16-byte aligned); arrays 0 .. n_read-1 are read and
+ * arrays 0 .. n_write-1 are also written in place, 1 <= n_write <= n_read <= 7 (OPTIMI_ERR_ARG
+ * otherwise) - AdamW with Kahan summation is 5 read / 4 written, Lion 4 / 3, StableAdamW's two
+ * passes 3 / 2 and 4 / 2, Adan 7 / 6.  The launch is the optimizers' own: the same kernel,
+ * 64-lane tiles, streaming loads, write-through tile stores, tensor table / chunk map and
+ * occupancy throttle as a 16-bit step with n_read + n_write streams, so bytes moved / duration
+ * is the ceiling of that access mix on the machine at hand.  `granules` = 0 takes the occupancy
+ * the library would choose for such a step; 1 .. 51 requests that many 1280-byte LDS granules
+ * per workgroup instead (a CU holds floor(128 / granules) workgroups).  `flags`: 0, OPTIMI_COLD,
+ * OPTIMI_PROBE_SCRAMBLE.  Every stored vector depends on every loaded one (as the parameter, the
+ * first array an optimizer stores, depends on all of its inputs).  The written arrays keep their
+ * contents: each is stored back as it was read (the bandwidth of this memory depends a little on
+ * the data, so the probe leaves the step's own data in place); with OPTIMI_PROBE_SCRAMBLE they
+ * are overwritten with a mix of everything that was read, which is how the tests see what the
+ * probe touched. */
+int optimi_hip_stream_probe(optimi_group* group, int n_tensors, void* const* const* arrays, const int64_t* bytes,
+                            int n_read, int n_write, int granules, uint32_t flags, optimi_stream_t stream);
 
 /* Measurement aid (no counterpart in the reference): the number of step, reduction and probe
  * kernels this library has launched in this process so far, every entry point and every thread

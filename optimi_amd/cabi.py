@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(HERE, "liboptimi_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
 KAHAN, UPDATE, DECOUPLE_WD, ADAM_WD, DECOUPLE_LR, DAMPENING, RECTIFY, LOOKAHEAD, COLD = 1, 2, 4, 8, 16, 32, 64, 128, 256
+PROBE_SCRAMBLE = 512
 
 _p, _pp, _i, _i64, _u32, _d = C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_int64, C.c_uint32, C.c_double
 _i64p = C.POINTER(C.c_int64)
@@ -49,6 +50,7 @@ PROTOTYPES = {
     "optimi_hip_radam_single": (_i, [_p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_ranger_single": (_i, [_p, _p, _p, _p, _p, _p, _i64, _i, _d, _d, _d, _d, _d, _d, _d, _d, _u32, _p]),
     "optimi_hip_copy_probe": (_i, [_p, _p, _i64, _p]),
+    "optimi_hip_stream_probe": (_i, [_p, _i, _pp, _i64p, _i, _i, _i, _u32, _p]),
     "optimi_hip_launch_count": (_i64, []),
 }
 
@@ -85,6 +87,14 @@ def ptr_array(ptrs):
     """A C array of void* from an iterable of integer addresses (None = NULL)."""
     ptrs = list(ptrs)
     return (C.c_void_p * max(len(ptrs), 1))(*ptrs)
+
+
+def ptr_table(columns):
+    """A C array of pointers to C arrays of void*: ``columns[a][i]`` is the address of array ``a`` of
+    tensor ``i``.  Returns the table and the inner arrays, which the caller keeps alive for the call."""
+    inner = [ptr_array(col) for col in columns]
+    table = (C.c_void_p * max(len(inner), 1))(*[C.cast(col, C.c_void_p).value for col in inner])
+    return table, inner
 
 
 def i64_array(vals):

@@ -28,9 +28,11 @@
 #include <cstdlib>
 #include <atomic>
 #include <cstring>
+#include <initializer_list>
 #include <mutex>
 #include <new>
 #include <type_traits>
+#include <utility>
 #include <vector>
 
 #include "optimi_hip.h"
@@ -530,6 +532,53 @@ struct AdanOp {
     }
   }
 };
+
+struct ProbeScalars {
+  uint32_t salt, mask;
+};
+
+// Measurement aid, not an optimizer: the memory traffic of a step with NR arrays read and the
+// first NW of them written in place, and no floating-point work.  It runs through the very
+// kernel, tiles, loads, stores, tables and occupancy throttle the optimizers use, so what it
+// reaches is the ceiling of that access mix on the machine at hand: AdamW with Kahan is 5 read /
+// 4 written, Lion 4 / 3, StableAdamW's passes 3 / 2 and 4 / 2, Adan 7 / 6.  The 16-byte vectors
+// pass through as raw bits (the F32 policy neither converts nor rounds).  Every stored vector
+// depends on every loaded one - as the parameter, the first array an optimizer stores, depends on
+// all of its inputs - so no load can be dropped and a lane's stores follow all of its loads.
+// What is stored is the array's own content xor (a mix of everything loaded & mask): the mask is 0
+// unless the caller asks for scrambling, so the arrays keep their bits (the bandwidth of this
+// memory depends a little on the data, and a probe that filled the arrays with noise would be
+// measured on other data than the step it stands for); the compiler cannot know that.
+template <int NR, int NW>
+struct ProbeOp {
+  using DT = F32;
+  using F32Partner = ProbeOp<NR, NW>;
+  using Scalars = ProbeScalars;
+  static constexpr bool kProbe = true;
+  static constexpr int kArrays = kMaxArrays;
+  static constexpr uint32_t kLoad = (1u << NR) - 1u;
+  static constexpr uint32_t kStore = (1u << NW) - 1u;
+  static constexpr bool kReduce = false;
+  static_assert(NW >= 1 && NW <= NR && NR <= kMaxArrays, "written arrays are among the read ones");
+  __device__ static __forceinline__ void prepare(Scalars&, int) {}
+  __device__ static __forceinline__ void elem(f32x2* x, const Scalars& s, f32x2&) {
+    uint32_t d0 = s.salt, d1 = s.salt;
+#pragma unroll
+    for (int a = 0; a < NR; ++a) {
+      d0 ^= __float_as_uint(x[a].x);
+      d1 ^= __float_as_uint(x[a].y);
+    }
+#pragma unroll
+    for (int a = 0; a < NW; ++a)
+      x[a] = f32x2{__uint_as_float(__float_as_uint(x[a].x) ^ ((d0 + (uint32_t)a) & s.mask)),
+                   __uint_as_float(__float_as_uint(x[a].y) ^ ((d1 + (uint32_t)a) & s.mask))};
+  }
+};
+
+template <class Op, class = void>
+struct is_probe : std::false_type {};
+template <class Op>
+struct is_probe<Op, std::enable_if_t<Op::kProbe>> : std::true_type {};
 
 // ------------------------------------------------------------------------------------
 // the streaming kernel
@@ -1129,11 +1178,17 @@ struct LaunchShape {
 // sits a little lower: the table as it is for 7 streams and more (no extra workgroup for
 // launches under kLongLaunch), 9 granules instead of 8 for 5 and 6 streams (measured on
 // per-tensor launches over tensors that are cold when revisited, 4 M to 45 M elements).
+// `request` > 0: the caller names the granules itself (the traffic probe's sweep).
 template <class Op>
-LaunchShape launch_shape(int64_t workgroups, bool few, bool misaligned) {
+LaunchShape launch_shape(int64_t workgroups, bool few, bool misaligned, int request = 0) {
   constexpr int streams = (popcount(Op::kLoad) + popcount(Op::kStore)) * kUnroll;
-  constexpr bool f32 = std::is_same<typename Op::DT, F32>::value;
+  // the traffic probe stands in for a 16-bit step with as many streams, whatever its own vector type
+  constexpr bool f32 = std::is_same<typename Op::DT, F32>::value && !is_probe<Op>::value;
   LaunchShape shape;
+  if (request > 0) {
+    shape.lds = (unsigned)((request > 51 ? 51 : request) * kLdsGranule - 128);
+    return shape;
+  }
   int granules = kBestGranules[streams < kMaxStreams ? streams : kMaxStreams];
   if (f32 && streams == 11) granules = 17;
   if (!few && !f32 && streams >= 7 && workgroups < kLongLaunch) granules -= 1;
@@ -1178,9 +1233,9 @@ std::atomic<int64_t> kernel_launches{0};  // every kernel this library has launc
 // `s_f32`: the same scalars formed for fp32 tensors; read only when the plan is a mixed list.
 template <class Op>
 void launch_list(optimi_group* g, const ListPlan& plan, const typename Op::Scalars& s, hipStream_t stream,
-                 double* partials = nullptr, const typename Op::Scalars* s_f32 = nullptr) {
+                 double* partials = nullptr, const typename Op::Scalars* s_f32 = nullptr, int granules = 0) {
   const int64_t workgroups = plan.n_chunks * kSub;
-  const LaunchShape shape = launch_shape<Op>(workgroups, plan.few, plan.misaligned);
+  const LaunchShape shape = launch_shape<Op>(workgroups, plan.few, plan.misaligned, granules);
   ++kernel_launches;
   if constexpr (!std::is_same<typename Op::DT, F32>::value) {
     if (plan.mixed) {
@@ -1715,6 +1770,57 @@ int ranger_list(optimi_group* g, int n_tensors, void* const* param, const void* 
   return finish_list(g, plan, stream);
 }
 
+// Calls fn(ProbeOp<NR, NW>{}) for 1 <= NW <= NR <= kMaxArrays.
+template <int NR, class Fn, int... W>
+void probe_pick_write(int n_write, Fn&& fn, std::integer_sequence<int, W...>) {
+  (void)std::initializer_list<int>{(n_write == W + 1 ? (fn(ProbeOp<NR, W + 1>{}), 0) : 0)...};
+}
+template <class Fn, int... R>
+void probe_pick(int n_read, int n_write, Fn&& fn, std::integer_sequence<int, R...>) {
+  (void)std::initializer_list<int>{
+      (n_read == R + 1 ? (probe_pick_write<R + 1>(n_write, fn, std::make_integer_sequence<int, R + 1>{}), 0) : 0)...};
+}
+
+int probe_list(optimi_group* g, int n_tensors, void* const* const* arrays, const int64_t* bytes, int n_read, int n_write,
+               int granules, uint32_t flags, hipStream_t stream) {
+  if (!g) return OPTIMI_ERR_NULL;
+  if (n_tensors < 0) return OPTIMI_ERR_SIZE;
+  if (n_write < 1 || n_write > n_read || n_read > kMaxArrays) return OPTIMI_ERR_ARG;
+  if (granules < 0 || granules > 51) return OPTIMI_ERR_ARG;
+  if (n_tensors > 0 && (!arrays || !bytes)) return OPTIMI_ERR_NULL;
+  const void* const* lists[kMaxArrays] = {};
+  std::vector<int64_t> numel;
+  try {
+    numel.resize((size_t)n_tensors);
+  } catch (const std::bad_alloc&) {
+    return OPTIMI_ERR_NOMEM;
+  }
+  for (int a = 0; a < n_read; ++a) {
+    if (n_tensors > 0 && !arrays[a]) return OPTIMI_ERR_NULL;
+    lists[a] = (const void* const*)arrays[a];
+  }
+  for (int t = 0; t < n_tensors; ++t) {
+    if (bytes[t] < 0 || bytes[t] % 16) return OPTIMI_ERR_SIZE;
+    numel[(size_t)t] = bytes[t] / 4;
+    for (int a = 0; a < n_read; ++a) {
+      if (!arrays[a][t] && bytes[t] > 0) return OPTIMI_ERR_NULL;
+      if ((uintptr_t)arrays[a][t] % 16) return OPTIMI_ERR_ALIGN;
+    }
+  }
+  ListPlan plan;
+  int rc = plan_list(g, n_tensors, lists, kMaxArrays, (1u << n_read) - 1u, 0u, numel.data(), nullptr, OPTIMI_F32, flags, stream,
+                     &plan);
+  if (rc) return rc;
+  if (plan.n_chunks == 0) return 0;
+  ProbeScalars s;
+  s.salt = 0x9e3779b9u;
+  s.mask = (flags & OPTIMI_PROBE_SCRAMBLE) ? 0xffffffffu : 0u;
+  probe_pick(n_read, n_write,
+             [&](auto op) { launch_list<decltype(op)>(g, plan, s, stream, nullptr, nullptr, granules); },
+             std::make_integer_sequence<int, kMaxArrays>{});
+  return finish_list(g, plan, stream);
+}
+
 }  // namespace
 
 // ------------------------------------------------------------------------------------
@@ -2090,6 +2196,11 @@ int optimi_hip_copy_probe(void* dst, const void* src, int64_t bytes, optimi_stre
   copy_probe_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream_>>>((u32x4*)dst, (const u32x4*)src, n_vec);
   HIP_TRY(hipGetLastError());
   return 0;
+}
+
+int optimi_hip_stream_probe(optimi_group* g, int n_tensors, void* const* const* arrays, const int64_t* bytes, int n_read,
+                            int n_write, int granules, uint32_t flags, optimi_stream_t stream) {
+  return probe_list(g, n_tensors, arrays, bytes, n_read, n_write, granules, flags, (hipStream_t)stream);
 }
 
 int64_t optimi_hip_launch_count(void) { return kernel_launches.load(); }

@@ -39,7 +39,8 @@ def test_error_strings_and_constants():
     # the flag values the Python side uses are the header's
     text = open(HEADER).read()
     for name, val in (("KAHAN", cabi.KAHAN), ("UPDATE", cabi.UPDATE), ("DECOUPLE_WD", cabi.DECOUPLE_WD),
-                      ("ADAM_WD", cabi.ADAM_WD), ("DECOUPLE_LR", cabi.DECOUPLE_LR)):
+                      ("ADAM_WD", cabi.ADAM_WD), ("DECOUPLE_LR", cabi.DECOUPLE_LR), ("COLD", cabi.COLD),
+                      ("PROBE_SCRAMBLE", cabi.PROBE_SCRAMBLE)):
         assert re.search(rf"OPTIMI_{name}\s*=\s*{val}\b", text), name
 
 
@@ -58,3 +59,22 @@ def test_null_group_is_rejected_before_any_device_work():
     assert L.optimi_hip_adam_single(None, None, None, None, None, 8, cabi.F32, 1e-3, 0.1, 0.9, 0.1, 0.0, 1e-6, 2, None) == -1
     assert L.optimi_hip_adam_single(None, None, None, None, None, 0, cabi.F32, 1e-3, 0.1, 0.9, 0.1, 0.0, 1e-6, 2, None) == 0
     assert L.optimi_hip_copy_probe(None, None, 16, None) == -1
+
+
+def test_stream_probe_rejects_bad_mixes_before_any_device_work():
+    L = cabi.lib()
+    table, keep = cabi.ptr_table([[None]] * 7)
+    sizes = cabi.i64_array([0])
+    assert L.optimi_hip_stream_probe(None, 1, table, sizes, 5, 4, 0, 0, None) == -1          # no group
+    fake = ctypes.c_void_p(1)  # never dereferenced: the mix is checked first
+    for n_read, n_write in ((0, 0), (3, 0), (3, 4), (8, 2), (-1, 1)):
+        assert L.optimi_hip_stream_probe(fake, 1, table, sizes, n_read, n_write, 0, 0, None) == -7, (n_read, n_write)
+    assert L.optimi_hip_stream_probe(fake, 1, table, sizes, 5, 4, 52, 0, None) == -7          # more LDS than a workgroup may ask for
+    assert L.optimi_hip_stream_probe(fake, 1, table, sizes, 5, 4, -1, 0, None) == -7
+    assert L.optimi_hip_stream_probe(fake, -1, table, sizes, 5, 4, 0, 0, None) == -2
+    assert L.optimi_hip_stream_probe(fake, 1, None, sizes, 5, 4, 0, 0, None) == -1
+    assert L.optimi_hip_stream_probe(fake, 1, table, cabi.i64_array([24]), 5, 4, 0, 0, None) == -2   # not whole vectors
+    assert L.optimi_hip_stream_probe(fake, 1, table, cabi.i64_array([32]), 5, 4, 0, 0, None) == -1   # null array with bytes
+    off, keep2 = cabi.ptr_table([[4096 + 8]] * 7)
+    assert L.optimi_hip_stream_probe(fake, 1, off, cabi.i64_array([32]), 5, 4, 0, 0, None) == -4     # off the 16-byte grid
+    del keep, keep2
