@@ -67,7 +67,8 @@ enum optimi_status {
   OPTIMI_ERR_DEVICE = -5,    /* group used on a device other than the one it was made on */
   OPTIMI_ERR_NOMEM = -6,     /* host allocation failed                             */
   OPTIMI_ERR_ARG = -7,       /* inconsistent scalar argument (e.g. max_lr <= 0 with OPTIMI_DECOUPLE_LR) */
-  OPTIMI_ERR_LIMIT = -8      /* numel above OPTIMI_NOALLOC_MAX_NUMEL in the allocation-free entry point */
+  OPTIMI_ERR_LIMIT = -8,     /* numel above OPTIMI_NOALLOC_MAX_NUMEL in the allocation-free entry point */
+  OPTIMI_ERR_CAPTURE = -9    /* `stream` is capturing a HIP graph and the list's tables would have to be uploaded */
 };
 
 /* Text for a status returned by any function of this header. */
@@ -87,7 +88,11 @@ int64_t optimi_hip_chunk_elems(int dtype);
  * re-uploaded only when a pointer or size differs from the previous call; a list of at most
  * 16 tensors needs no tables at all (its pointers travel as kernel arguments).  A group
  * belongs to the device that was current when it was created and must be used by
- * one thread and one stream at a time.  (No counterpart in the reference: it plays
+ * one thread and one stream at a time.  Under HIP graph capture a whole-list call uploads
+ * nothing and keeps the group's own stream bookkeeping out of the graph: a list of more than 16
+ * tensors must have been stepped once, with the same pointers and sizes, before the capture
+ * begins (and that step must have completed), otherwise the call returns OPTIMI_ERR_CAPTURE;
+ * StableAdamW's reduction scratch must have been sized by such a step as well.  (No counterpart in the reference: it plays
  * the role of the Python loop in optimi/adam.py:551-583.)
  * ------------------------------------------------------------------------------- */
 typedef struct optimi_group optimi_group;
@@ -301,6 +306,20 @@ int optimi_hip_stream_probe(optimi_group* group, int n_tensors, void* const* con
  * counted (the small copy that brings a changed tensor table to the device is not).  Tests and
  * benchmarks take differences of it to see how many launches a step costs. */
 int64_t optimi_hip_launch_count(void);
+
+/* The largest total size, in bytes, of the arrays a whole-list launch works on for which the
+ * launch, unless marked OPTIMI_COLD, reads them with cached loads (see OPTIMI_COLD).  A caller that
+ * steps several lists per optimizer step compares the sum over all of them with this and passes
+ * OPTIMI_COLD when the sum is larger: a short list of a large model has left the cache by the
+ * time it is stepped again.  No counterpart in the reference. */
+int64_t optimi_hip_resident_bytes(void);
+
+/* Measurement aids (no counterpart in the reference), counted like optimi_hip_launch_count:
+ * how many tensor tables and chunk maps have been copied to the device (a list of more than 16
+ * tensors whose pointers and sizes are those of the group's previous call uploads nothing), and
+ * how many of the kernels launched for lists read their tensors with cached loads. */
+int64_t optimi_hip_upload_count(void);
+int64_t optimi_hip_resident_launch_count(void);
 
 #ifdef __cplusplus
 }

@@ -33,17 +33,19 @@ def ext():
     return _ext
 
 
-_groups: dict = {}
+_thread = threading.local()
 
 
 def default_group(device: torch.device, dtype: torch.dtype, tag: str = ""):
-    """A per-thread launch workspace for functional calls that bring none of their own."""
-    key = (threading.get_ident(), device.type, device.index, dtype, tag)
-    grp = _groups.get(key)
+    """A per-thread launch workspace for functional calls that bring none of their own; it goes
+    when its thread does."""
+    groups = _thread.__dict__.setdefault("groups", {})
+    key = (device.type, device.index, dtype, tag)
+    grp = groups.get(key)
     if grp is None:
         with torch.cuda.device(device):
             grp = ext().Group()
-        _groups[key] = grp
+        groups[key] = grp
     return grp
 
 

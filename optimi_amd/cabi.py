@@ -52,6 +52,9 @@ PROTOTYPES = {
     "optimi_hip_copy_probe": (_i, [_p, _p, _i64, _p]),
     "optimi_hip_stream_probe": (_i, [_p, _i, _pp, _i64p, _i, _i, _i, _u32, _p]),
     "optimi_hip_launch_count": (_i64, []),
+    "optimi_hip_resident_bytes": (_i64, []),
+    "optimi_hip_upload_count": (_i64, []),
+    "optimi_hip_resident_launch_count": (_i64, []),
 }
 
 _lib = None

@@ -909,6 +909,8 @@ struct DeviceBuf {
   }
 };
 
+std::atomic<int64_t> table_uploads{0};  // tensor tables and chunk maps copied to the device so far
+
 struct StagingSlot {
   void* host = nullptr;
   size_t cap = 0;
@@ -963,9 +965,21 @@ int staged_upload(optimi_group* g, void* dst, const void* src, size_t bytes, hip
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipEventRecord(slot.done, stream));
   slot.in_flight = true;
+  ++table_uploads;
   return 0;
 }
 
+
+// Whether work put on `stream` is being recorded into a HIP graph instead of run.  A capture
+// must not see the group's own bookkeeping: an event recorded inside a capture cannot be waited
+// for or synchronised on by eager work afterwards, and a copy recorded from the pinned staging
+// ring would replay from a slot that later uploads overwrite.
+int stream_capturing(hipStream_t stream, bool* capturing) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  HIP_TRY(hipStreamIsCapturing(stream, &status));
+  *capturing = status != hipStreamCaptureStatusNone;
+  return 0;
+}
 
 // A list whose arrays add up to at most this many bytes stays in the 256 MB last-level cache
 // from one optimizer step to the next (measured: cached loads beat `nt` loads up to 270 MB of
@@ -1058,11 +1072,19 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
   }
 
   // a group moved to another stream must not overwrite tables a previous launch still reads
-  if (g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
+  // (a capturing stream uploads nothing, see below, and takes no part in the group's events)
+  bool capturing = false;
+  rc = stream_capturing(stream, &capturing);
+  if (rc) return rc;
+  if (!capturing && g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
 
   // the chunk map is a function of where every tensor's chunks start and of how many there are
   bool same_map = g->map_first.size() == (size_t)n_tensors + 1 && g->map_first[(size_t)n_tensors] == n_chunks;
   for (int t = 0; same_map && t < n_tensors; ++t) same_map = g->map_first[(size_t)t] == fresh[(size_t)t].first_chunk;
+  if (capturing && ((!same_map && n_chunks > 0) ||
+                    !(g->host_table.size() == fresh.size() &&
+                      std::memcmp(g->host_table.data(), fresh.data(), sizeof(TensorEntry) * fresh.size()) == 0)))
+    return OPTIMI_ERR_CAPTURE;  // the tables must be on the device before the capture begins
   if (!same_map && n_chunks > 0) {
     g->map_first.clear();  // the cached map is void until the new one is on its way
     try {
@@ -1104,6 +1126,10 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
 
 int note_launch(optimi_group* g, hipStream_t stream) {
   HIP_TRY(hipGetLastError());
+  bool capturing = false;
+  int rc = stream_capturing(stream, &capturing);
+  if (rc) return rc;
+  if (capturing) return 0;  // the graph orders its own nodes; the group's event stays an eager one
   if (!g->last_launch) HIP_TRY(hipEventCreateWithFlags(&g->last_launch, hipEventDisableTiming));
   HIP_TRY(hipEventRecord(g->last_launch, stream));
   g->last_stream = stream;
@@ -1229,6 +1255,7 @@ LaunchShape launch_shape(int64_t workgroups, bool few, bool misaligned, int requ
 const FewTable kNoTable = {};
 
 std::atomic<int64_t> kernel_launches{0};  // every kernel this library has launched in this process
+std::atomic<int64_t> resident_launches{0};  // list launches among them that read with cached loads
 
 // `s_f32`: the same scalars formed for fp32 tensors; read only when the plan is a mixed list.
 template <class Op>
@@ -1237,6 +1264,7 @@ void launch_list(optimi_group* g, const ListPlan& plan, const typename Op::Scala
   const int64_t workgroups = plan.n_chunks * kSub;
   const LaunchShape shape = launch_shape<Op>(workgroups, plan.few, plan.misaligned, granules);
   ++kernel_launches;
+  if (plan.resident) ++resident_launches;
   if constexpr (!std::is_same<typename Op::DT, F32>::value) {
     if (plan.mixed) {
       if (plan.few)
@@ -1656,7 +1684,12 @@ int stableadamw_list(optimi_group* g, int n_tensors, void* const* param, const v
   if (rc) return rc;
   if (plan.n_chunks == 0) return 0;
   // the reduction scratch is the group's: a previous launch on another stream may still read it
-  if (plan.few && g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
+  if (plan.few && g->launched && g->last_stream != stream) {
+    bool capturing = false;
+    rc = stream_capturing(stream, &capturing);
+    if (rc) return rc;
+    if (!capturing) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
+  }
   TensorEntry none;
   std::memset(&none, 0, sizeof(none));
   rc = dtype == OPTIMI_BF16
@@ -1838,6 +1871,7 @@ const char* optimi_hip_error_string(int status) {
     case OPTIMI_ERR_DEVICE: return "optimi_hip: group used on a different device than it was created on";
     case OPTIMI_ERR_NOMEM: return "optimi_hip: host allocation failed";
     case OPTIMI_ERR_ARG: return "optimi_hip: inconsistent scalar argument";
+    case OPTIMI_ERR_CAPTURE: return "optimi_hip: the stream is capturing a HIP graph and this list's tables are not on the device yet (step the same list once before the capture)";
     case OPTIMI_ERR_LIMIT: return "optimi_hip: tensor has more elements than the fixed scratch of the allocation-free entry point covers (OPTIMI_NOALLOC_MAX_NUMEL)";
     default: break;
   }
@@ -2009,7 +2043,12 @@ int optimi_hip_stableadamw_single(optimi_group* g, void* param, const void* grad
   int dev = 0;
   HIP_TRY(hipGetDevice(&dev));
   if (dev != g->device) return OPTIMI_ERR_DEVICE;
-  if (g->launched && g->last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
+  if (g->launched && g->last_stream != stream) {
+    bool capturing = false;
+    rc = stream_capturing(stream, &capturing);
+    if (rc) return rc;
+    if (!capturing) HIP_TRY(hipStreamWaitEvent(stream, g->last_launch, 0));
+  }
   rc = dtype == OPTIMI_BF16
            ? stable_group_run<BF16>(nullptr, g, e, dtype, lr, beta1_comp, beta2_hat, beta2_comp, weight_decay, eps, max_lr, flags, stream)
        : dtype == OPTIMI_F16
@@ -2204,5 +2243,11 @@ int optimi_hip_stream_probe(optimi_group* g, int n_tensors, void* const* const* 
 }
 
 int64_t optimi_hip_launch_count(void) { return kernel_launches.load(); }
+
+int64_t optimi_hip_resident_bytes(void) { return kResidentBytes; }
+
+int64_t optimi_hip_upload_count(void) { return table_uploads.load(); }
+
+int64_t optimi_hip_resident_launch_count(void) { return resident_launches.load(); }
 
 }  // extern "C"

@@ -551,7 +551,12 @@ void check_hip(hipError_t err, const char* what) {
 class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
  public:
   ReleaseQueue(int64_t max_numel, int64_t max_tensors, int64_t max_total)
-      : max_numel_(max_numel), max_tensors_(max_tensors), max_total_(max_total) {}
+      : max_numel_(max_numel), max_tensors_(max_tensors), max_total_(max_total) {
+    if (max_tensors > 0 && max_tensors < (1 << 20)) {
+      batch_.reserve((size_t)max_tensors);
+      seen_.reserve((size_t)max_tensors);
+    }
+  }
   ~ReleaseQueue() {
     // steps still parked are dropped, never launched from a destructor (the device may be gone);
     // their step counters have advanced, so say so
@@ -561,8 +566,16 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
                    batch_.size());
   }
 
-  bool wants(const StepCall& c) const {
-    return c.param().numel() <= max_numel_ && torch::autograd::get_current_graph_task_id() != -1;
+  // Parks the step if a backward pass is running and the tensor is small enough, and makes sure
+  // the pass ends with a flush; `c` is moved from only when it was parked.
+  bool try_park(StepCall&& c) {
+    if (c.param().numel() > max_numel_) return false;
+    const int task = torch::autograd::get_current_graph_task_id();
+    if (task == -1) return false;
+    std::lock_guard<std::recursive_mutex> lock(mutex_);
+    add(std::move(c));
+    schedule(task);
+    return true;
   }
   int64_t pending() {
     std::lock_guard<std::recursive_mutex> lock(mutex_);
@@ -572,10 +585,9 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
   int64_t launches() const { return launches_; }
   int64_t launched_steps() const { return launched_steps_; }
 
-  // Makes sure the running backward pass ends with a flush.
-  void schedule() {
+  // Makes sure the running backward pass `task` ends with a flush.
+  void schedule(int task) {
     std::lock_guard<std::recursive_mutex> lock(mutex_);
-    const int task = torch::autograd::get_current_graph_task_id();
     if (task == -1 || task == scheduled_task_) return;
     std::weak_ptr<ReleaseQueue> weak = weak_from_this();
     torch::autograd::Engine::get_default_engine().queue_callback([weak] {
@@ -597,6 +609,7 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
     if (batch_.empty()) {
       stream_ = stream;
       low_dtype_ = at::kFloat;
+      batch_.reserve((size_t)(max_tensors_ > 0 && max_tensors_ < 4096 ? max_tensors_ : 4096));  // flush() took the old storage along
     }
     if (c.param().scalar_type() != at::kFloat) low_dtype_ = c.param().scalar_type();
     total_ += c.param().numel() * (int64_t)c.param().element_size();
@@ -696,11 +709,7 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
 // Parks the step when there is a queue, a backward pass is running and the tensor is small
 // enough, otherwise launches it.  Returns whether the step was parked.
 bool submit(StepCall&& c, ReleaseQueue* queue, Group* stable_group = nullptr) {
-  if (queue && queue->wants(c)) {
-    queue->add(std::move(c));
-    queue->schedule();
-    return true;
-  }
+  if (queue && queue->try_park(std::move(c))) return true;
   launch_now(c, stable_group);
   return false;
 }
@@ -874,15 +883,26 @@ class ReleaseHookCore {
   // calls this whenever its state or groups are replaced wholesale (load_state_dict).
   void invalidate() {
     entries_.clear();
+    workspaces_.clear();  // keyed by group dicts that may be gone now
+    hyper_cache_.clear();
     rebind();
   }
 
 
   void call(const py::handle& param_h) {
     TORCH_CHECK(THPVariable_Check(param_h.ptr()), "optimi_amd: the gradient release hook takes the parameter");
-    py::object optimizer = optimizer_();
-    TORCH_CHECK(!optimizer.is_none(), "optimi_amd: the optimizer of this gradient release hook no longer exists");
-    if (any_step_hooks()) {
+    PyObject* opt_ptr = PyWeakref_GetObject(optimizer_.ptr());  // borrowed
+    TORCH_CHECK(opt_ptr && opt_ptr != Py_None, "optimi_amd: the optimizer of this gradient release hook no longer exists");
+    py::object optimizer = py::reinterpret_borrow<py::object>(opt_ptr);
+    // What is the same for every parameter of a backward pass - whether step hooks are registered,
+    // whether the pass only accumulates - is looked up once per pass (outside a pass: every call).
+    const int task = torch::autograd::get_current_graph_task_id();
+    if (task == -1 || task != pass_task_) {
+      pass_hooks_ = any_step_hooks();
+      pass_update_ = !truthy(py::reinterpret_steal<py::object>(attr(opt_ptr, k_.accumulation)).ptr());
+      pass_task_ = task;
+    }
+    if (pass_hooks_) {
       optimizer.attr(k_.release)(param_h);
       return;
     }
@@ -892,11 +912,10 @@ class ReleaseHookCore {
     const at::Tensor g = p.grad();
     TORCH_CHECK(g.defined(), "optimi_amd: the gradient release hook ran on a parameter without a gradient");
     at::NoGradGuard no_grad;
-    const bool update = !truthy(py::reinterpret_steal<py::object>(attr(optimizer.ptr(), k_.accumulation)).ptr());
     PyObject* grp = e->group.ptr();
-    StepCall c = pack(*e, Hyper{}, p, grad_like(p, g), num_or_zero(grp));
+    StepCall c = pack(*e, Hyper{}, p, grad_like(p, g), momentum_of(grp));
     validate_call(c);  // before the counter moves: a rejected step leaves the state as it was
-    submit(set_hyper(std::move(c), read_hyper(grp, has_step_ ? tick(e->step) : 0, update)), queue_.get(), e->workspace);
+    submit(set_hyper(std::move(c), hyper_for(grp, has_step_ ? tick(e->step) : 0, pass_update_)), queue_.get(), e->workspace);
     p.mutable_grad().reset();  // param.grad = None
   }
 
@@ -905,7 +924,10 @@ class ReleaseHookCore {
   // the group's step counter, forms the scalars and launches one list per device.
   // Returns false, having done nothing, when the group has not been set up yet (the first step
   // goes through Python, which resolves the backend) - the caller then takes the Python path.
-  bool step_group(const py::dict& group) {
+  // `cold`: the optimizer's tensors do not fit the last-level cache as a whole, so even a short
+  // list (the few norm weights and biases of a no-decay group beside 100 GB of matrices) has left
+  // it since the previous step and is read with streaming loads (OPTIMI_COLD).
+  bool step_group(const py::dict& group, bool cold) {
     PyObject* grp = group.ptr();
     if (!flag(grp, k_.setup) || item(grp, k_.triton) != Py_True) return false;
     py::object optimizer = optimizer_();
@@ -920,7 +942,7 @@ class ReleaseHookCore {
       Entry* e;
     };
     std::vector<Item> items;
-    const double momentum = num_or_zero(grp);
+    const double momentum = momentum_of(grp);
     const Py_ssize_t n_params = PyList_GET_SIZE(plist);
     items.reserve((size_t)n_params);
     for (Py_ssize_t i = 0; i < n_params; ++i) {
@@ -945,7 +967,7 @@ class ReleaseHookCore {
       t = tick(THPVariable_Unpack(step));
     }
     if (items.empty()) return true;
-    const Hyper h = read_hyper(grp, t, true);
+    const Hyper h = hyper_for(grp, t, true);
 
     // pass 2: one launch per device, in order of first appearance.  fp32 parameters and the
     // parameters of one 16-bit dtype go together; a group that holds bf16 and fp16 gets a launch for each.
@@ -987,9 +1009,13 @@ class ReleaseHookCore {
         }
       }
       c10::hip::HIPGuardMasqueradingAsCUDA guard(p0.device());
-      std::unique_ptr<Group>& slot = workspaces_[{(int)p0.device().index(), (int)low}];
+      // one workspace per parameter group (and device, and 16-bit dtype): its device tables then hold
+      // this group's list from one step to the next and are uploaded once, however many groups
+      // the optimizer steps in between
+      std::unique_ptr<Group>& slot = workspaces_[{grp, (int)p0.device().index(), (int)low}];
       if (!slot) slot = std::make_unique<Group>();
-      launch_list(kind_, slot->get(), (int)numel.size(), ptr, numel.data(), dtypes.data(), h.s, h.flags,
+      launch_list(kind_, slot->get(), (int)numel.size(), ptr, numel.data(), dtypes.data(), h.s,
+                  h.flags | (cold ? (uint32_t)OPTIMI_COLD : 0u),
                   c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(p0.device().index()).stream());
     }
     return true;
@@ -1003,6 +1029,8 @@ class ReleaseHookCore {
     PyObject* ids[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
     PyObject* step_id = nullptr;
     bool release = false;  // made for the gradient-release hook (group and step counter cached too)
+    uint64_t state_version = 0;    // the state dict's version tag when the cached tensors were last checked against it
+    bool checked_release = false;  // that check covered the group and the step counter too
     std::optional<at::Tensor> t[5];
     at::Tensor step;
     explicit Entry(const at::Tensor& p) : param(p.getIntrusivePtr()) {}
@@ -1048,7 +1076,44 @@ class ReleaseHookCore {
   }
 
   // SGD keeps a momentum buffer in its state even when momentum is 0; it is not passed then
-  double num_or_zero(PyObject* grp) const { return kind_ == SGD ? num(grp, k_.momentum) : 1.0; }
+  double momentum_of(PyObject* grp) const { return kind_ == SGD ? num(grp, k_.momentum) : 1.0; }
+
+  // A dict's version tag changes whenever the dict is modified (a key added or removed, a value
+  // replaced by another object), so an unchanged tag means that everything read from the dict
+  // before still holds.  0 = not available on this interpreter: nothing is cached then.
+  static uint64_t dict_version(PyObject* dict) {
+#if PY_VERSION_HEX < 0x030C0000
+    return ((PyDictObject*)dict)->ma_version_tag;
+#else
+    (void)dict;
+    return 0;
+#endif
+  }
+
+  // The step scalars of a group at step count `t`.  Every parameter of a group shares them, so
+  // they are formed once (a dozen dict reads and two or three pow() calls) and reused for as long as
+  // the group dict is unmodified and the step count and the kind of step are the same - a
+  // scheduler that rewrites group["lr"] changes the dict's version tag and is seen at once.
+  const Hyper& hyper_for(PyObject* grp, int64_t t, bool update) {
+    const uint64_t version = dict_version(grp);
+    HyperSlot* slot = nullptr;
+    for (HyperSlot& s : hyper_cache_)
+      if (s.group == grp) slot = &s;
+    if (!slot) {
+      hyper_cache_.emplace_back();
+      slot = &hyper_cache_.back();
+      slot->group = grp;
+      slot->version = 0;
+    }
+    if (version == 0 || slot->version != version || slot->t != t || slot->update != update) {
+      slot->version = 0;  // void while it is being rebuilt (read_hyper may throw)
+      slot->h = read_hyper(grp, t, update);
+      slot->t = t;
+      slot->update = update;
+      slot->version = version;
+    }
+    return slot->h;
+  }
 
   Hyper read_hyper(PyObject* grp, int64_t t, bool update) const {
     switch (kind_) {
@@ -1128,14 +1193,20 @@ class ReleaseHookCore {
 
   // every cached tensor is still the object the state dict holds
   // (`release`: also the group and the per-parameter step counter that gradient release keeps there)
-  bool valid(const Entry& e, bool release = true) const {
+  // (an unmodified state dict - same version tag as when it was last checked - needs no look-ups)
+  bool valid(Entry& e, bool release = true) const {
     PyObject* st = e.state.ptr();
+    if (release && !e.release) return false;
+    const uint64_t version = dict_version(st);
+    if (version != 0 && version == e.state_version && e.checked_release >= release) return true;
     for (size_t i = 0; i < state_keys_.size(); ++i)
       if (PyDict_GetItemWithError(st, state_keys_[i].ptr()) != e.ids[i]) return false;
-    if (!release) return true;
-    if (!e.release) return false;
-    if (PyDict_GetItemWithError(st, k_.group.ptr()) != e.group.ptr()) return false;
-    if (has_step_ && PyDict_GetItemWithError(st, k_.step.ptr()) != e.step_id) return false;
+    if (release) {
+      if (PyDict_GetItemWithError(st, k_.group.ptr()) != e.group.ptr()) return false;
+      if (has_step_ && PyDict_GetItemWithError(st, k_.step.ptr()) != e.step_id) return false;
+    }
+    e.state_version = version;
+    e.checked_release = release;
     return true;
   }
 
@@ -1182,10 +1253,27 @@ class ReleaseHookCore {
   std::vector<py::str> state_keys_;
   std::vector<py::object> hook_tables_;
   std::unordered_map<c10::TensorImpl*, Entry> entries_;
-  struct PairHash {
-    size_t operator()(const std::pair<int, int>& k) const { return std::hash<int64_t>()(((int64_t)k.first << 32) ^ (int64_t)k.second); }
+  struct HyperSlot {
+    PyObject* group = nullptr;
+    uint64_t version = 0;
+    int64_t t = 0;
+    bool update = false;
+    Hyper h;
   };
-  std::unordered_map<std::pair<int, int>, std::unique_ptr<Group>, PairHash> workspaces_;  // (device, 16-bit dtype of the list or float) -> tables
+  std::vector<HyperSlot> hyper_cache_;  // one slot per parameter group seen
+  int pass_task_ = -1;                  // the backward pass pass_hooks_ and pass_update_ were read in
+  bool pass_hooks_ = false, pass_update_ = true;
+  struct WorkspaceKey {
+    PyObject* group;  // the parameter group's dict (an address only, never dereferenced)
+    int device, low;  // the list's device and its 16-bit dtype (float for an all-fp32 list)
+    bool operator==(const WorkspaceKey& o) const { return group == o.group && device == o.device && low == o.low; }
+  };
+  struct WorkspaceHash {
+    size_t operator()(const WorkspaceKey& k) const {
+      return std::hash<const void*>()(k.group) ^ (std::hash<int64_t>()(((int64_t)k.device << 32) ^ (int64_t)k.low) * 0x9e3779b97f4a7c15ull);
+    }
+  };
+  std::unordered_map<WorkspaceKey, std::unique_ptr<Group>, WorkspaceHash> workspaces_;  // the launch tables of each list
 };
 
 // What is registered on the parameters: a handle that does not own the hook, so that
@@ -1216,12 +1304,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.attr("DAMPENING") = (uint32_t)OPTIMI_DAMPENING;
   mod.attr("RECTIFY") = (uint32_t)OPTIMI_RECTIFY;
   mod.attr("LOOKAHEAD") = (uint32_t)OPTIMI_LOOKAHEAD;
+  mod.attr("COLD") = (uint32_t)OPTIMI_COLD;
+  mod.def("resident_bytes", &optimi_hip_resident_bytes);
   mod.def("abi_version", &optimi_hip_version);
   py::class_<Group>(mod, "Group").def(py::init<>());
   py::class_<ReleaseHookCore, std::shared_ptr<ReleaseHookCore>>(mod, "ReleaseHookCore")
       .def(py::init<const py::object&, int, std::shared_ptr<ReleaseQueue>>(), py::arg("optimizer"), py::arg("kind"), py::arg("queue"))
       .def("invalidate", &ReleaseHookCore::invalidate)
-      .def("step_group", &ReleaseHookCore::step_group)
+      .def("step_group", &ReleaseHookCore::step_group, py::arg("group"), py::arg("cold") = false)
       .def("__call__", &ReleaseHookCore::call);
   py::class_<ReleaseHook>(mod, "ReleaseHook")
       .def(py::init<const std::shared_ptr<ReleaseHookCore>&>())

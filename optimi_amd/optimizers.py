@@ -62,6 +62,11 @@ class OptimiOptimizer(Optimizer):
     # that up to _QUEUE_MAX_BYTES of gradients (plus one tensor) stay alive until their launch.
     # Set on the instance, or on the class, before prepare_for_gradient_release.
     native_step = True                      # False: walk the parameters in Python on every step (same results)
+    # How a whole-group step reads its tensors.  None: decided from the optimizer's size - when all its
+    # parameters, gradients and states together fit the GPU's last-level cache, a step finds them there
+    # from the step before and reads them with cached loads; otherwise every list, also the few norm
+    # weights of a small group, is streamed.  True / False force the one or the other.  Results are the same.
+    resident_lists: bool | None = None
     gradient_release_coalesce = 1 << 26
     _QUEUE_MAX_TENSORS = 1024               # parked steps per launch
     _QUEUE_MAX_BYTES = 128 << 20            # bytes of parked gradients kept alive at most
@@ -102,6 +107,7 @@ class OptimiOptimizer(Optimizer):
         self._hip_groups: dict = {}
         self._release_queue = None
         self._release_hook = None
+        self._cold = None
 
         if self.defaults["gradient_release"]:
             if self.defaults["foreach"]:  # optimi/optimizer.py:65-68
@@ -120,6 +126,7 @@ class OptimiOptimizer(Optimizer):
         state.pop("_hip_groups", None)
         state.pop("_release_queue", None)
         state.pop("_release_hook", None)
+        state.pop("_cold", None)
         return state
 
     def __setstate__(self, state):
@@ -127,6 +134,7 @@ class OptimiOptimizer(Optimizer):
         self.__dict__.setdefault("_hip_groups", {})
         self.__dict__.setdefault("_release_queue", None)
         self.__dict__.setdefault("_release_hook", None)
+        self.__dict__["_cold"] = None
         self._invalidate_release_cache()
         self.__dict__.setdefault("_optimizer_accumulation", False)
 
@@ -230,9 +238,10 @@ class OptimiOptimizer(Optimizer):
         if param is None:
             self._flush_release()
             driver = self._driver() if self.native_step else None
+            cold = self._lists_are_cold()
             for group in self.param_groups:
                 # after a group's first step the whole walk over its parameters is native
-                if driver is not None and group["setup"] and driver.step_group(group):
+                if driver is not None and group["setup"] and driver.step_group(group, cold):
                     continue
                 params = self._collect(group)
                 if params and not group["triton"]:
@@ -339,8 +348,29 @@ class OptimiOptimizer(Optimizer):
         return backend.ext().ReleaseHook(self._driver())
 
     def _invalidate_release_cache(self):
+        self.__dict__["_cold"] = None
+        self.__dict__.get("_hip_groups", {}).clear()  # keyed by group dicts that may be gone now
         if self.__dict__.get("_release_hook") is not None:
             self._release_hook.invalidate()
+
+    def _lists_are_cold(self) -> bool:
+        """Whether a whole-group step must take its tensors for gone from the last-level cache since the
+        previous step: they are when everything the optimizer touches in a step is larger than that cache."""
+        if self.resident_lists is not None:
+            return not self.resident_lists
+        if self._cold is None:
+            total = 0
+            for group in self.param_groups:
+                for p in group["params"]:
+                    arrays = 2 + len(self._moment_keys) + (1 if p.dtype in _LOW_PRECISION else 0)
+                    total += p.numel() * p.element_size() * arrays
+            self._cold = total > backend.ext().resident_bytes()
+        return self._cold
+
+    def _workspaces(self, group: dict) -> dict:
+        """The launch workspaces of one parameter group: its device tables then keep this group's list
+        from one step to the next, however many other groups the optimizer steps in between."""
+        return self._hip_groups.setdefault(id(group), {})
 
     def load_state_dict(self, state_dict):
         super().load_state_dict(state_dict)
@@ -436,7 +466,7 @@ class Adam(OptimiOptimizer):
                lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"], weight_decay=group["weight_decay"],
                eps=group["eps"], step=step, decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"],
                max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
-               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
+               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
 
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
@@ -514,7 +544,7 @@ class Lion(OptimiOptimizer):
         F.lion(params, grads, _col(states, "exp_avg"), _col(states, "kahan_comp"), lr=group["lr"], beta1=group["beta1"],
                beta2=group["beta2"], weight_decay=group["weight_decay"], decouple_lr=group["decouple_lr"],
                max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
-               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
+               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
 
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
@@ -589,11 +619,11 @@ class StableAdamW(OptimiOptimizer):
                       weight_decay=group["weight_decay"], eps=group["eps"], step=step, decouple_lr=group["decouple_lr"],
                       max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
                       gradient_release=gradient_release, optimizer_accumulation=accumulate, mean_squares=None,
-                      _groups=self._hip_groups)
+                      _groups=self._workspaces(group), _cold=self._lists_are_cold())
 
 
     def _release_workspace(self, param):
-        return F._workspace(self._hip_groups, param.device, param.dtype, "stableadamw_single")
+        return F._workspace(self._hip_groups.setdefault("per_tensor", {}), param.device, param.dtype, "stableadamw_single")
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
         grp = self._release_workspace(param)
@@ -664,7 +694,7 @@ class Adan(OptimiOptimizer):
                beta2=group["beta2"], beta3=group["beta3"], eps=group["eps"], weight_decay=group["weight_decay"],
                step=step, decouple_lr=group["decouple_lr"], max_lr=group["max_lr"], kahan_sum=group["kahan_sum"],
                foreach=False, triton=True, gradient_release=gradient_release,
-               optimizer_accumulation=accumulate, _groups=self._hip_groups)
+               optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
         # adam_wd is not forwarded, as in step() above
@@ -746,7 +776,7 @@ class SGD(OptimiOptimizer):
               momentum=group["momentum"], weight_decay=group["weight_decay"], dampening=group["dampening"],
               decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"], max_lr=group["max_lr"],
               kahan_sum=group["kahan_sum"], foreach=False, triton=True, gradient_release=gradient_release,
-              optimizer_accumulation=accumulate, _groups=self._hip_groups)
+              optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
         return ext.sgd_release(param, grad, state["exp_avg"], state["kahan_comp"], group["lr"], group["momentum"],
@@ -800,7 +830,7 @@ class RAdam(OptimiOptimizer):
                 lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"], weight_decay=group["weight_decay"],
                 eps=group["eps"], step=step, decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"],
                 max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
-                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._hip_groups)
+                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
         return ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], None, state["kahan_comp"], state["step"],
@@ -862,7 +892,7 @@ class Ranger(OptimiOptimizer):
                  weight_decay=group["weight_decay"], eps=group["eps"], k=group["k"], alpha=group["alpha"], step=step,
                  decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"], max_lr=group["max_lr"],
                  kahan_sum=group["kahan_sum"], foreach=False, triton=True, gradient_release=gradient_release,
-                 optimizer_accumulation=accumulate, _groups=self._hip_groups)
+                 optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
         return ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], state["la_param"], state["kahan_comp"],

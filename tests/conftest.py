@@ -20,3 +20,21 @@ def hip_device():
     if not torch.cuda.is_available():
         pytest.skip("no HIP device")
     return torch.device("cuda:0")
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The fp32 fixtures are compared with a stated floor; what they measure with no floor at all is
+    printed here, so that a regression in it is visible in the log of every run."""
+    try:
+        import golden_util as G
+    except Exception:
+        return
+    if not G.FP32_WORST:
+        return
+    tr = terminalreporter
+    tr.write_sep("-", "fp32 results against the reference's fixtures, no floor: worst |a-b|/max(|a|,|b|) (fp32 ulps, abs) at")
+    for opt in sorted(G.FP32_WORST):
+        for kind in ("param", "state"):
+            if kind in G.FP32_WORST[opt]:
+                rel, ulps, absd, where = G.FP32_WORST[opt][kind]
+                tr.write_line(f"  {opt:12s} {kind:5s} {rel:9.3e}  ({ulps:5.1f} ulp, abs {absd:8.2e})  {where}")

@@ -128,6 +128,27 @@ def fp32_rel_err(a: torch.Tensor, b: torch.Tensor, floor: float) -> torch.Tensor
     return (a - b).abs() / torch.maximum(torch.maximum(a.abs(), b.abs()), torch.tensor(floor, dtype=torch.float64))
 
 
+# worst fp32 disagreement seen in this run with no floor applied: optimizer -> {"param" | "state": (rel, ulps, abs)}
+FP32_WORST: dict = {}
+
+
+def note_fp32_error(name: str, key: str, got: torch.Tensor, want: torch.Tensor):
+    a, b = got.detach().cpu().float().flatten(), want.detach().cpu().float().flatten()
+    fin = torch.isfinite(a) & torch.isfinite(b)
+    a, b = a[fin], b[fin]
+    if a.numel() == 0:
+        return
+    diff = (a.double() - b.double()).abs()
+    big = torch.maximum(a.abs(), b.abs()).double()
+    rel = torch.where(big > 0, diff / big.clamp_min(1e-300), torch.zeros_like(diff))
+    i = int(rel.argmax())
+    ulp = torch.exp2(torch.floor(torch.log2(big[i].clamp_min(2.0**-126))) - 23)
+    kind = "param" if (".param." in key or ".la_param." in key) else "state"
+    slot = FP32_WORST.setdefault(name.split("_")[0], {})
+    if float(rel[i]) > slot.get(kind, (-1.0,))[0]:
+        slot[kind] = (float(rel[i]), float(diff[i] / ulp), float(diff[i]), f"{name} {key}")
+
+
 def assert_bits_equal(got: torch.Tensor, want: torch.Tensor, what: str):
     a = got.detach().cpu().contiguous()
     b = want.detach().cpu().contiguous()

@@ -30,7 +30,7 @@ def test_error_strings_and_constants():
     L = cabi.lib()
     assert L.optimi_hip_version() >= 1000
     assert L.optimi_hip_error_string(0) == b"success"
-    for code in range(-8, 0):
+    for code in range(-9, 0):
         msg = L.optimi_hip_error_string(code)
         assert msg.startswith(b"optimi_hip:"), (code, msg)
     assert L.optimi_hip_chunk_elems(cabi.BF16) == 8192
@@ -78,3 +78,19 @@ def test_stream_probe_rejects_bad_mixes_before_any_device_work():
     off, keep2 = cabi.ptr_table([[4096 + 8]] * 7)
     assert L.optimi_hip_stream_probe(fake, 1, off, cabi.i64_array([32]), 5, 4, 0, 0, None) == -4     # off the 16-byte grid
     del keep, keep2
+
+
+def test_noalloc_limit_matches_its_scratch():
+    """A tensor of exactly OPTIMI_NOALLOC_MAX_NUMEL elements needs exactly as many pass-1 partials as the
+    fixed scratch holds behind its 256-byte head: a chunk of 16 KiB per array is shared by 16 one-wavefront
+    workgroups of 1 KiB, each of which leaves one double."""
+    text = open(HEADER).read()
+    scratch = re.search(r"#define OPTIMI_NOALLOC_SCRATCH_BYTES \((\d+)u \* (\d+)u \* (\d+)u \+ (\d+)u\)", text)
+    a, b, c, head = (int(x) for x in scratch.groups())
+    limits = re.search(r"#define OPTIMI_NOALLOC_MAX_NUMEL\(dtype\) \(\(dtype\) == OPTIMI_F32 \? \(int64_t\)(\d+) : \(int64_t\)(\d+)\)", text)
+    max_f32, max_low = (int(x) for x in limits.groups())
+    partials = (a * b * c + head - 256) // 8
+    L = cabi.lib()
+    for dtype, limit in ((cabi.F32, max_f32), (cabi.BF16, max_low), (cabi.F16, max_low)):
+        chunk = L.optimi_hip_chunk_elems(dtype)
+        assert limit % chunk == 0 and limit // chunk * 16 == partials, (dtype, limit, chunk, partials)

@@ -11,8 +11,11 @@ is only faithfully rounded, so fp32 cannot be bit-exact.  Where the reference's 
 is not uniform (the scalar remainder loop of ATen's ``add_(x, alpha=...)``, used by SGD, RAdam,
 Ranger and L2 decay) the last ``numel % 32`` elements are left out.  The floor covers elements that
 cancel towards zero: 1e-2 for parameters (ten steps move a parameter by up to about 10 * lr, so
-its rounding error is judged against that distance, i.e. |a-b| <= 1e-8 near zero) and the
-tensor's RMS for the moment states.
+its rounding error is judged against that distance, i.e. |a-b| <= 1e-8 near zero) for StableAdamW's
+parameters, a tenth of the tensor's RMS (about 2e-3) for every other optimizer's, and the tensor's RMS
+for the moment states.  The worst error with no floor at all - |a-b| / max(|a|, |b|), and in fp32 ulps -
+is collected per optimizer and printed at the end of the run (tests/conftest.py), so that a change in
+it shows in the log even while the floored comparison still passes.
 """
 
 import functools
@@ -25,7 +28,7 @@ import golden_util as G
 pytestmark = pytest.mark.gpu
 
 FP32_REL = 1e-6
-FP32_FLOOR_PARAM = 1e-2
+FP32_FLOOR_PARAM = 1e-2  # StableAdamW; every other optimizer is held to a tenth of the tensor's RMS (about 2e-3)
 
 
 def compare_snapshot(name, key, got, want, param_want=None):
@@ -43,8 +46,11 @@ def compare_snapshot(name, key, got, want, param_want=None):
         else:
             assert int(ulp.max()) <= 1, f"{name} {key}: max {int(ulp.max())} ulp"
     else:
-        floor = FP32_FLOOR_PARAM if (".param." in key or ".la_param." in key) else max(float(want.double().pow(2).mean().sqrt()), 1e-30)
+        rms = max(float(want.double().pow(2).mean().sqrt()), 1e-30)
+        is_param = ".param." in key or ".la_param." in key
+        floor = (FP32_FLOOR_PARAM if "stableadamw" in name else 0.1 * rms) if is_param else rms
         rel = G.fp32_rel_err(got, want, floor)
+        G.note_fp32_error(name, key, got, want)  # the unfloored figures, for the summary at the end of the run
         assert float(rel.max()) <= FP32_REL, f"{name} {key}: rel err {float(rel.max())}"
 
 
@@ -55,6 +61,22 @@ def test_fixture(name, multi, hip_device):
 
     fx = G.load(name)
     out = G.replay(name, fx, functools.partial(HipRun, multi=multi), device=hip_device)
+    wanted = [k for k in fx if k.startswith("out.")]
+    assert sorted(out) == sorted(wanted)
+    for key in wanted:
+        step, _, idx = key.split(".")[1], key.split(".")[2], key.split(".")[3]
+        compare_snapshot(name, key, out[key], fx[key], fx.get(f"out.{step}.param.{idx}"))
+
+
+@pytest.mark.parametrize("multi", [True, False], ids=["multi", "single"])
+@pytest.mark.parametrize("name", G.case_names())
+def test_fixture_through_a_driver_that_owes_the_oracle_nothing(name, multi, hip_device):
+    """The same fixtures through ``PlainHipRun``: its state creation and scalar prologue share no
+    code with ``oracle/`` (``HipRun`` inherits both from the oracle's driver)."""
+    from hip_engine import PlainHipRun
+
+    fx = G.load(name)
+    out = G.replay(name, fx, functools.partial(PlainHipRun, multi=multi), device=hip_device)
     wanted = [k for k in fx if k.startswith("out.")]
     assert sorted(out) == sorted(wanted)
     for key in wanted:

@@ -63,7 +63,6 @@ def test_two_calls_in_a_row_second_smaller(hip_device, dtype):
     # partials than the first one wrote
     first = _compare(3 * 8192 + 1000 + 3, dtype, hip_device, 1, SCALARS, flags, group, big_grad=True)
     second = _compare(300, dtype, hip_device, 2, SCALARS, flags, group, big_grad=True)
-    # the step really clipped: with lr' < lr the parameter moved less than the unclipped Adam step would move it
     assert first[0].numel() > second[0].numel()
     # a third, larger call after the small one
     _compare(70_000, dtype, hip_device, 3, SCALARS, flags, group)
@@ -110,3 +109,81 @@ def test_limit_and_argument_errors(hip_device):
     assert fn(a, a, a, a, a, 0, cabi.BF16, *SCALARS, flags, stream) == 0
     torch.cuda.synchronize()
     assert float(t.float().abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_the_step_really_clips(hip_device, dtype):
+    """With gradients far above sqrt(exp_avg_sq) the RMS is well above 1, so the learning rate the step
+    uses is lr / RMS: the parameter must move by clearly less than the same Adam step without clipping
+    moves it (optimi_hip_adam_single on the same inputs and scalars, no decay in either).  A run in
+    which the partial sums or the per-tensor scalars were not read back from the scratch would step
+    with the plain lr - or with garbage - and fail here."""
+    numel = 50_000
+    scalars = SCALARS[:4] + (0.0,) + SCALARS[5:]  # no weight decay
+    start = _inputs(numel, dtype, hip_device, 21, big_grad=True)
+    clipped = [t.clone() for t in start]
+    plain = [t.clone() for t in start]
+    flags = cabi.UPDATE
+    _step("optimi_hip_stableadamw_single_noalloc", None, clipped, numel, dtype, scalars, flags)
+    L = cabi.lib()
+    rc = L.optimi_hip_adam_single(plain[0].data_ptr(), plain[1].data_ptr(), plain[2].data_ptr(), plain[3].data_ptr(), None, numel,
+                                  DT[dtype], *scalars[:6], flags | cabi.DECOUPLE_WD, torch.cuda.current_stream().cuda_stream)
+    cabi.check(rc, "optimi_hip_adam_single")
+    torch.cuda.synchronize()
+    # the moments are the same step for both
+    assert torch.equal(clipped[2], plain[2]) and torch.equal(clipped[3], plain[3])
+    moved_clipped = (clipped[0].double() - start[0].double()).abs().mean().item()
+    moved_plain = (plain[0].double() - start[0].double()).abs().mean().item()
+    g, v_new = start[1].double(), clipped[3].double()
+    rms = (g * g / v_new.clamp_min(1e-12)).mean().sqrt().item()
+    assert rms > 2.0, rms
+    ratio = moved_clipped / moved_plain
+    if dtype == torch.float32:
+        assert 0.7 / rms < ratio < 1.3 / rms, (moved_clipped, moved_plain, rms)
+    else:  # a bf16 parameter moves in whole ulps, so only the direction of the effect is held
+        assert 0.0 < ratio < 0.6, (moved_clipped, moved_plain, rms)
+
+
+def test_no_device_memory_is_allocated(hip_device):
+    """What the entry point is for: after a first call (which looks the scratch's address up) calls of
+    any size below the limit leave the amount of free device memory exactly as it was - nothing is
+    allocated, nothing is freed - whereas the variant with a group grows the group's workspace."""
+    flags = cabi.KAHAN | cabi.UPDATE
+    sizes = [300, 3 * 8192 + 1000, 1 << 20, 5_000_000, 40_000_000, 17]
+    sets = {n: _inputs(n, torch.bfloat16, hip_device, 30 + i, big_grad=True) for i, n in enumerate(sizes)}
+    _step("optimi_hip_stableadamw_single_noalloc", None, sets[300], 300, torch.bfloat16, SCALARS, flags)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        for n in sizes:
+            _step("optimi_hip_stableadamw_single_noalloc", None, sets[n], n, torch.bfloat16, SCALARS, flags)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    # the same calls through a group do allocate (its workspace grows to the largest tensor's partials)
+    group = cabi.Group()
+    for n in sizes:
+        _step("optimi_hip_stableadamw_single", group, sets[n], n, torch.bfloat16, SCALARS, flags)
+    torch.cuda.synchronize()
+    free_group, _ = torch.cuda.mem_get_info()
+    assert free_group < free_after
+    group.close()
+
+
+def test_exactly_the_largest_tensor(hip_device):
+    """OPTIMI_NOALLOC_MAX_NUMEL(bf16) = 2^28 elements: every one of the scratch's 524,288 partials is
+    written and read; the result equals the group variant's."""
+    numel = 268435456
+    group = cabi.Group()
+    gen = torch.Generator(device=hip_device).manual_seed(9)
+    want = [torch.empty(numel, dtype=torch.float32, device=hip_device).normal_(0, s, generator=gen).bfloat16()
+            for s in (0.02, 3e-2, 1e-3, 1e-3, 1e-5)]
+    want[3].abs_().mul_(1e-3)
+    got = [t.clone() for t in want]
+    flags = cabi.KAHAN | cabi.UPDATE
+    _step("optimi_hip_stableadamw_single", group, want, numel, torch.bfloat16, SCALARS, flags)
+    _step("optimi_hip_stableadamw_single_noalloc", None, got, numel, torch.bfloat16, SCALARS, flags)
+    torch.cuda.synchronize()
+    for name, a, b in zip(NAMES, got, want):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"{name} differs at the size limit"
+    group.close()
