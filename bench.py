@@ -333,22 +333,19 @@ def release_bench(workload, args, steps, warmup):
         def backward(ctx, grad_out):
             return tuple(g.view(g.shape) for g in grads)  # fresh tensor objects, so autograd adopts them as .grad
 
-    # what the same backward pass costs when the hook only frees the gradient: the share of the
-    # autograd engine and of this harness in the figures below
-    handles = [p.register_post_accumulate_grad_hook(lambda p: setattr(p, "grad", None)) for p in params]
-    for _ in range(2):
-        Feed.apply(*params).backward()
-    def empty_hook_pass_ms(n=8):
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(n):
-            Feed.apply(*params).backward()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / n * 1e3
+    def timed_passes(run, n):
+        """Wall time of each of n backward passes, in ms (the device is idle at both ends of each)."""
+        out = []
+        for i in range(n):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            run(i)
+            torch.cuda.synchronize()
+            out.append((time.perf_counter() - t0) * 1e3)
+        return out
 
-    floor_before_ms = empty_hook_pass_ms()
-    for h in handles:
-        h.remove()
+    def median(xs):
+        return sorted(xs)[len(xs) // 2]
 
     kwargs = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
     opt = optimi_amd.AdamW(params, gradient_release=True, **kwargs)
@@ -375,15 +372,24 @@ def release_bench(workload, args, steps, warmup):
     full = sum(1 for i in range(steps) if (warmup + i + 1) % 4 == 0)
     algo_bytes = n_params * (18.0 * full + 10.0 * (steps - full))
     achieved = algo_bytes / elapsed / 1e9
+    # What the optimizer adds to a backward pass: the same passes with a hook that only frees the gradient
+    # (the autograd engine's and this harness's share) in alternation with passes that step - four of the
+    # one, one accumulation cycle of the other, three times over, each pass timed on its own; medians, since the
+    # host's speed drifts over a run and a garbage collection now and then lands in a pass.
+    empty_ms, stepping_ms = [], []
+    for block in range(3):
+        optimi_amd.remove_gradient_release(model)
+        handles = [p.register_post_accumulate_grad_hook(lambda p: setattr(p, "grad", None)) for p in params]
+        Feed.apply(*params).backward()
+        empty_ms += timed_passes(lambda i: Feed.apply(*params).backward(), 4)
+        for h in handles:
+            h.remove()
+        optimi_amd.prepare_for_gradient_release(model, opt)
+        one_pass(2)
+        stepping_ms += timed_passes(lambda i: one_pass(warmup + steps + i), 4)
     optimi_amd.remove_gradient_release(model)
-    # the same empty-hook passes once more afterwards: the host's speed drifts over a run, and the smaller of
-    # the two figures is the one the optimizer's share is measured against (so that share is not flattered)
-    handles = [p.register_post_accumulate_grad_hook(lambda p: setattr(p, "grad", None)) for p in params]
-    Feed.apply(*params).backward()
-    floor_after_ms = empty_hook_pass_ms()
-    for h in handles:
-        h.remove()
-    floor_ms = min(floor_before_ms, floor_after_ms)
+    floor_ms = median(empty_ms)
+    over_floor_us = (median(stepping_ms) - floor_ms) * 1e3 / len(shapes)
     out = {
         "metric": "gradient-release tensor-steps/s (AdamW bf16 Kahan, accumulation_steps=4)",
         "value": len(shapes) * steps / elapsed, "unit": "tensor-steps/s", "n_gpus": 1, "steps": steps,
@@ -391,8 +397,9 @@ def release_bench(workload, args, steps, warmup):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": workload, "optimizer": "AdamW", "n_tensors": len(shapes), "n_params": n_params,
                    "coalesce": opt.gradient_release_coalesce, "empty_hook_pass_ms": floor_ms,
-                   "empty_hook_pass_ms_before_and_after": [floor_before_ms, floor_after_ms],
-                   "us_per_tensor_over_empty_hook": (elapsed / steps * 1e3 - floor_ms) * 1e3 / len(shapes), "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()}},
+                   "stepping_pass_ms_beside_it": median(stepping_ms), "us_per_tensor_over_empty_hook": over_floor_us,
+                   "over_empty_hook_from": "medians of 12 passes each, in alternating blocks of 4, every pass timed on its own",
+                   "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": None, "traffic_source": None,
                      "note": "wall clock over whole backward passes (hook dispatch included), launch-bound for small tensors; "
@@ -564,8 +571,8 @@ def cold_cache_bench(args, steps=100, evict_bytes=1 << 30):
             out[f"{policy}_{condition}"] = {"kernel_us": mean, "kernel_us_p50": us[len(us) // 2],
                                             "achieved_gbps": bytes_per_param * n_params / mean / 1e3,
                                             "frac": bytes_per_param * n_params / mean / 1e3 / HBM_PEAK_GBPS}
-    opt.resident_lists = None
-    out["library_default_reads_this_list_with"] = "streaming_loads" if opt._lists_are_cold() else "cached_loads"
+    opt.resident_lists = False
+    out["default"] = "streaming_loads (cached loads are opt-in: OptimiOptimizer.resident_lists / OPTIMI_RESIDENT)"
     del opt, params, grad_sets, src, dst
     return out
 

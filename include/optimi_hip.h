@@ -49,11 +49,14 @@ enum optimi_flags {
   OPTIMI_RECTIFY = 64,    /* RAdam/Ranger: rho > 5, take the rectified Adam step (optimi/radam.py:269-277) */
   OPTIMI_LOOKAHEAD = 128, /* Ranger: this step synchronises with the slow weights, step % k == 0
                              (optimi/ranger.py:452, 471)                                           */
-  OPTIMI_COLD = 256,      /* whole-list entry points: the tensors were not touched recently (they are a
-                             slice of a larger model, e.g. small tensors gathered during gradient
-                             release).  A hint: a short list otherwise counts as resident in the
-                             last-level cache and is read with cached instead of streaming loads.
-                             Results do not depend on it.  No counterpart in the reference.        */
+  OPTIMI_RESIDENT = 256,  /* whole-list entry points, a hint: the list was stepped a moment ago and nothing
+                             else has gone through the GPU's last-level cache since (a loop of optimizer
+                             steps with no forward or backward pass in between).  If its arrays also total
+                             at most optimi_hip_resident_bytes(), they are read with cached loads, which
+                             then hit.  Without the hint every list is read with streaming loads: after a
+                             backward pass nothing of it is left in the cache, and streaming loads are the
+                             faster ones on data that has to come from memory.  Results do not depend on
+                             it.  No counterpart in the reference.                                  */
   OPTIMI_PROBE_SCRAMBLE = 512 /* optimi_hip_stream_probe only: the written arrays get new bits (a mix of
                              everything that was read) instead of keeping theirs                    */
 };
@@ -291,7 +294,7 @@ int optimi_hip_copy_probe(void* dst, const void* src, int64_t bytes, optimi_stre
  * occupancy throttle as a 16-bit step with n_read + n_write streams, so bytes moved / duration
  * is the ceiling of that access mix on the machine at hand.  `granules` = 0 takes the occupancy
  * the library would choose for such a step; 1 .. 51 requests that many 1280-byte LDS granules
- * per workgroup instead (a CU holds floor(128 / granules) workgroups).  `flags`: 0, OPTIMI_COLD,
+ * per workgroup instead (a CU holds floor(128 / granules) workgroups).  `flags`: 0, OPTIMI_RESIDENT,
  * OPTIMI_PROBE_SCRAMBLE.  Every stored vector depends on every loaded one (as the parameter, the
  * first array an optimizer stores, depends on all of its inputs).  The written arrays keep their
  * contents: each is stored back as it was read (the bandwidth of this memory depends a little on
@@ -307,11 +310,10 @@ int optimi_hip_stream_probe(optimi_group* group, int n_tensors, void* const* con
  * benchmarks take differences of it to see how many launches a step costs. */
 int64_t optimi_hip_launch_count(void);
 
-/* The largest total size, in bytes, of the arrays a whole-list launch works on for which the
- * launch, unless marked OPTIMI_COLD, reads them with cached loads (see OPTIMI_COLD).  A caller that
- * steps several lists per optimizer step compares the sum over all of them with this and passes
- * OPTIMI_COLD when the sum is larger: a short list of a large model has left the cache by the
- * time it is stepped again.  No counterpart in the reference. */
+/* The largest total size, in bytes, of the arrays a whole-list launch works on for which
+ * OPTIMI_RESIDENT is honoured (see there).  A caller that steps several lists per optimizer step
+ * compares the sum over all of them with this before passing the hint: a short list of a large
+ * model has left the cache by the time it is stepped again.  No counterpart in the reference. */
 int64_t optimi_hip_resident_bytes(void);
 
 /* Measurement aids (no counterpart in the reference), counted like optimi_hip_launch_count:

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "liboptimi_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
-KAHAN, UPDATE, DECOUPLE_WD, ADAM_WD, DECOUPLE_LR, DAMPENING, RECTIFY, LOOKAHEAD, COLD = 1, 2, 4, 8, 16, 32, 64, 128, 256
+KAHAN, UPDATE, DECOUPLE_WD, ADAM_WD, DECOUPLE_LR, DAMPENING, RECTIFY, LOOKAHEAD, RESIDENT = 1, 2, 4, 8, 16, 32, 64, 128, 256
 PROBE_SCRAMBLE = 512
 
 _p, _pp, _i, _i64, _u32, _d = C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_int64, C.c_uint32, C.c_double

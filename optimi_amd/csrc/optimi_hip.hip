@@ -60,7 +60,7 @@ constexpr int kSub = kChunkBytes / (kThreads * kUnroll * 16);  // workgroups per
 static_assert(kSub >= 1 && kSub * kThreads * kUnroll * 16 == kChunkBytes, "workgroup tile must divide the chunk");
 static_assert(kThreads % 64 == 0 && kThreads <= 1024, "whole wavefronts");
 constexpr int kReduceThreads = 1024;      // lanes of the per-tensor finalize workgroup
-constexpr int kAbiVersion = 1002;
+constexpr int kAbiVersion = 1003;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -982,11 +982,14 @@ int stream_capturing(hipStream_t stream, bool* capturing) {
 }
 
 // A list whose arrays add up to at most this many bytes stays in the 256 MB last-level cache
-// from one optimizer step to the next (measured: cached loads beat `nt` loads up to 270 MB of
-// arrays and lose from 335 MB on).  Such a launch - unless the caller marks it OPTIMI_COLD -
-// uses cached loads.  Per-tensor entry points never take this path: they step one tensor of a
-// larger model, which was last touched a whole backward pass ago (measured on tensors that are
-// cold when revisited: `nt` loads are 6-8 % faster there than cached ones).
+// from one optimizer step to the next when nothing else runs in between (measured: cached loads
+// beat `nt` loads up to 270 MB of arrays and lose from 335 MB on).  A caller that knows this is so
+// says OPTIMI_RESIDENT, and such a launch then uses cached loads: 1 % faster than streaming ones
+// on a 269 MB fp32 list stepped back to back.  It is a hint to opt in with, not the default: a
+// training loop runs a forward and a backward pass between two optimizer steps, after which the
+// list has to come from memory, and there streaming loads are the faster ones (the same list with
+// 2 GiB moved through the caches before every step: 71.5 us streaming, 77.2 us cached).
+// Per-tensor entry points never take this path: they step one tensor of a larger model.
 constexpr int64_t kResidentBytes = (int64_t)288 << 20;
 
 // What one list launch works on, as the entry points hand it to the launchers.
@@ -1063,7 +1066,7 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
     if (!(entries[t].flags & optimi_tables::kEntryVec)) off_grid += b;
   }
   plan->misaligned = 2 * off_grid > bytes;
-  plan->resident = !(flags & OPTIMI_COLD) && bytes <= kResidentBytes;
+  plan->resident = (flags & OPTIMI_RESIDENT) && bytes <= kResidentBytes;
   if (plan->resident)
     for (int t = 0; t < n_tensors; ++t) entries[t].flags |= optimi_tables::kEntryCached;
   if (plan->few) {

@@ -11,9 +11,11 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/csrc/autograd/engine.h>
 #include <torch/csrc/autograd/graph_task.h>
+#include <torch/csrc/Exceptions.h>
 #include <torch/csrc/autograd/python_variable.h>
 #include <torch/extension.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstdio>
@@ -551,12 +553,8 @@ void check_hip(hipError_t err, const char* what) {
 class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
  public:
   ReleaseQueue(int64_t max_numel, int64_t max_tensors, int64_t max_total)
-      : max_numel_(max_numel), max_tensors_(max_tensors), max_total_(max_total) {
-    if (max_tensors > 0 && max_tensors < (1 << 20)) {
-      batch_.reserve((size_t)max_tensors);
-      seen_.reserve((size_t)max_tensors);
-    }
-  }
+      : max_numel_(max_numel), max_tensors_(max_tensors), max_total_(max_total),
+        seen_((size_t)(max_tensors > 0 && max_tensors < 4096 ? max_tensors : 4096)) {}
   ~ReleaseQueue() {
     // steps still parked are dropped, never launched from a destructor (the device may be gone);
     // their step counters have advanced, so say so
@@ -605,7 +603,7 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
   void add(StepCall&& c) {
     std::lock_guard<std::recursive_mutex> lock(mutex_);
     const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(c.param().device().index()).stream();
-    if (!batch_.empty() && (!same_run(c, stream) || seen_.count(c.param().data_ptr()))) flush();
+    if (!batch_.empty() && (!same_run(c, stream) || seen_.contains(c.param().data_ptr()))) flush();
     if (batch_.empty()) {
       stream_ = stream;
       low_dtype_ = at::kFloat;
@@ -663,9 +661,9 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
       // soon as this function returns: tell the caching allocator that another stream reads them.
       for (const StepCall& c : batch) c.t[1]->record_stream(current_stream);
     }
-    // OPTIMI_COLD: these tensors are a slice of a model whose backward pass has just streamed
-    // through the caches; a short list must not be taken for a small resident model
-    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtypes.data(), c0.s, c0.flags | OPTIMI_COLD, launch);
+    // never OPTIMI_RESIDENT: these tensors are a slice of a model whose backward pass has just
+    // gone through the caches
+    launch_list(c0.kind, slot->get(), n, ptr, numel.data(), dtypes.data(), c0.s, c0.flags, launch);
     ++launches_;
     launched_steps_ += n;
     if (launch != current) {
@@ -699,7 +697,50 @@ class ReleaseQueue : public std::enable_shared_from_this<ReleaseQueue> {
   int scheduled_task_ = -1;  // the backward pass that already carries the flush callback
   std::unordered_map<int, std::unique_ptr<Group>> groups_;
   std::vector<StepCall> batch_;
-  std::unordered_set<void*> seen_;
+  // The parameters parked so far (two steps of one parameter must not share a launch): a flat
+  // open-addressing table, because a node-based set pays an allocation for every parked step.
+  class PointerSet {
+   public:
+    explicit PointerSet(size_t expected) {
+      size_t cap = 64;
+      while (cap < 2 * expected) cap *= 2;
+      slots_.assign(cap, nullptr);
+    }
+    bool contains(const void* p) const {
+      for (size_t i = hash(p);; i = (i + 1) & (slots_.size() - 1)) {
+        if (slots_[i] == p) return true;
+        if (!slots_[i]) return false;
+      }
+    }
+    void insert(const void* p) {
+      if (2 * (count_ + 1) > slots_.size()) grow();
+      for (size_t i = hash(p);; i = (i + 1) & (slots_.size() - 1)) {
+        if (slots_[i] == p) return;
+        if (!slots_[i]) {
+          slots_[i] = p;
+          ++count_;
+          return;
+        }
+      }
+    }
+    void clear() {
+      if (count_) std::fill(slots_.begin(), slots_.end(), nullptr);
+      count_ = 0;
+    }
+
+   private:
+    size_t hash(const void* p) const { return (size_t)(((uintptr_t)p >> 4) * 0x9e3779b97f4a7c15ull >> 20) & (slots_.size() - 1); }
+    void grow() {
+      std::vector<const void*> old(2 * slots_.size(), nullptr);
+      old.swap(slots_);
+      count_ = 0;
+      for (const void* p : old)
+        if (p) insert(p);
+    }
+    std::vector<const void*> slots_;
+    size_t count_ = 0;
+  };
+  PointerSet seen_;
   int64_t total_ = 0;
   hipStream_t stream_ = nullptr;
   at::ScalarType low_dtype_ = at::kFloat;  // the 16-bit dtype among the parked tensors, float while there is none
@@ -924,10 +965,11 @@ class ReleaseHookCore {
   // the group's step counter, forms the scalars and launches one list per device.
   // Returns false, having done nothing, when the group has not been set up yet (the first step
   // goes through Python, which resolves the backend) - the caller then takes the Python path.
-  // `cold`: the optimizer's tensors do not fit the last-level cache as a whole, so even a short
-  // list (the few norm weights and biases of a no-decay group beside 100 GB of matrices) has left
-  // it since the previous step and is read with streaming loads (OPTIMI_COLD).
-  bool step_group(const py::dict& group, bool cold) {
+  // `resident`: the caller steps back to back, with nothing in between that would sweep the
+  // last-level cache, and everything the optimizer touches fits that cache - the list is then
+  // read with cached loads (OPTIMI_RESIDENT).  The size test is the caller's, over all groups: the
+  // few norm weights of a no-decay group beside 100 GB of matrices are not resident.
+  bool step_group(const py::dict& group, bool resident) {
     PyObject* grp = group.ptr();
     if (!flag(grp, k_.setup) || item(grp, k_.triton) != Py_True) return false;
     py::object optimizer = optimizer_();
@@ -1015,7 +1057,7 @@ class ReleaseHookCore {
       std::unique_ptr<Group>& slot = workspaces_[{grp, (int)p0.device().index(), (int)low}];
       if (!slot) slot = std::make_unique<Group>();
       launch_list(kind_, slot->get(), (int)numel.size(), ptr, numel.data(), dtypes.data(), h.s,
-                  h.flags | (cold ? (uint32_t)OPTIMI_COLD : 0u),
+                  h.flags | (resident ? (uint32_t)OPTIMI_RESIDENT : 0u),
                   c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(p0.device().index()).stream());
     }
     return true;
@@ -1279,18 +1321,49 @@ class ReleaseHookCore {
 // What is registered on the parameters: a handle that does not own the hook, so that
 // parameter -> hook -> cached state -> group -> parameter is not a cycle the garbage
 // collector cannot see.  The optimizer owns the ReleaseHookCore.
-class ReleaseHook {
- public:
-  explicit ReleaseHook(const std::shared_ptr<ReleaseHookCore>& core) : core_(core) {}
-  void call(const py::handle& param) {
-    std::shared_ptr<ReleaseHookCore> core = core_.lock();
-    TORCH_CHECK(core, "optimi_amd: the optimizer of this gradient release hook no longer exists");
-    core->call(param);
-  }
-
- private:
-  std::weak_ptr<ReleaseHookCore> core_;
+// The handle is a bare CPython type whose tp_call goes straight to ReleaseHookCore::call: the
+// autograd engine calls it once per parameter per backward pass, and a pybind11 method call
+// (overload resolution, argument casters) costs several hundred nanoseconds that a model with
+// thousands of small tensors pays thousands of times.
+struct ReleaseHookObject {
+  PyObject_HEAD
+  std::weak_ptr<ReleaseHookCore>* core;
 };
+
+PyObject* release_hook_call(PyObject* self, PyObject* args, PyObject* kwargs) {
+  HANDLE_TH_ERRORS
+  TORCH_CHECK(PyTuple_GET_SIZE(args) == 1 && (!kwargs || PyDict_GET_SIZE(kwargs) == 0),
+              "optimi_amd: the gradient release hook takes the parameter and nothing else");
+  std::shared_ptr<ReleaseHookCore> core = ((ReleaseHookObject*)self)->core->lock();
+  TORCH_CHECK(core, "optimi_amd: the optimizer of this gradient release hook no longer exists");
+  core->call(py::handle(PyTuple_GET_ITEM(args, 0)));
+  Py_RETURN_NONE;
+  END_HANDLE_TH_ERRORS
+}
+
+void release_hook_dealloc(PyObject* self) {
+  delete ((ReleaseHookObject*)self)->core;
+  Py_TYPE(self)->tp_free(self);
+}
+
+PyTypeObject ReleaseHookType = {PyVarObject_HEAD_INIT(nullptr, 0)};
+
+bool init_release_hook_type() {
+  ReleaseHookType.tp_name = "optimi_amd._C.ReleaseHook";
+  ReleaseHookType.tp_basicsize = sizeof(ReleaseHookObject);
+  ReleaseHookType.tp_flags = Py_TPFLAGS_DEFAULT;
+  ReleaseHookType.tp_doc = "post-accumulate-grad hook of one optimizer (callable with the parameter)";
+  ReleaseHookType.tp_call = release_hook_call;
+  ReleaseHookType.tp_dealloc = release_hook_dealloc;
+  return PyType_Ready(&ReleaseHookType) == 0;
+}
+
+py::object make_release_hook(const std::shared_ptr<ReleaseHookCore>& core) {
+  PyObject* obj = ReleaseHookType.tp_alloc(&ReleaseHookType, 0);
+  if (!obj) throw py::error_already_set();
+  ((ReleaseHookObject*)obj)->core = new std::weak_ptr<ReleaseHookCore>(core);
+  return py::reinterpret_steal<py::object>(obj);
+}
 
 }  // namespace
 
@@ -1304,18 +1377,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   mod.attr("DAMPENING") = (uint32_t)OPTIMI_DAMPENING;
   mod.attr("RECTIFY") = (uint32_t)OPTIMI_RECTIFY;
   mod.attr("LOOKAHEAD") = (uint32_t)OPTIMI_LOOKAHEAD;
-  mod.attr("COLD") = (uint32_t)OPTIMI_COLD;
+  mod.attr("RESIDENT") = (uint32_t)OPTIMI_RESIDENT;
   mod.def("resident_bytes", &optimi_hip_resident_bytes);
   mod.def("abi_version", &optimi_hip_version);
   py::class_<Group>(mod, "Group").def(py::init<>());
   py::class_<ReleaseHookCore, std::shared_ptr<ReleaseHookCore>>(mod, "ReleaseHookCore")
       .def(py::init<const py::object&, int, std::shared_ptr<ReleaseQueue>>(), py::arg("optimizer"), py::arg("kind"), py::arg("queue"))
       .def("invalidate", &ReleaseHookCore::invalidate)
-      .def("step_group", &ReleaseHookCore::step_group, py::arg("group"), py::arg("cold") = false)
+      .def("step_group", &ReleaseHookCore::step_group, py::arg("group"), py::arg("resident") = false)
       .def("__call__", &ReleaseHookCore::call);
-  py::class_<ReleaseHook>(mod, "ReleaseHook")
-      .def(py::init<const std::shared_ptr<ReleaseHookCore>&>())
-      .def("__call__", &ReleaseHook::call);
+  if (!init_release_hook_type()) throw py::error_already_set();
+  mod.def("ReleaseHook", &make_release_hook, py::arg("core"));
   mod.attr("KIND_ADAM") = (int)ADAM;
   mod.attr("KIND_LION") = (int)LION;
   mod.attr("KIND_STABLEADAMW") = (int)STABLEADAMW;

@@ -150,14 +150,14 @@ def adam(
     gradient_release: bool = False,
     optimizer_accumulation: bool = False,
     _groups=None,
-    _cold=False,
+    _resident=False,
 ):
     """Functional API to apply an Adam or AdamW optimization step (optimi/adam.py:213-309).
 
     Args mirror the reference: tensors (or lists of tensors) to update, their gradients and
     states, the raw hyper-parameters, and the int32 CPU ``step`` counter, which is advanced
     here.  ``_groups`` is an optional dict the caller owns in which launch workspaces are kept;
-    ``_cold`` marks a list that is part of something larger than the GPU's last-level cache.
+    ``_resident`` says that the list was stepped a moment ago and is still in the GPU's last-level cache.
     """
     _require_hip_backend(triton, foreach, gradient_release)
     ext = backend.ext()
@@ -171,7 +171,7 @@ def adam(
             weight_decay = 1 - (lr / max_lr) * weight_decay
         elif decouple_wd:
             weight_decay = 1 - lr * weight_decay
-    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, COLD=_cold,
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, RESIDENT=_resident,
                    DECOUPLE_WD=decouple_wd or decouple_lr)
     scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps, flags)
 
@@ -206,14 +206,14 @@ def adamw(
     gradient_release: bool = False,
     optimizer_accumulation: bool = False,
     _groups=None,
-    _cold=False,
+    _resident=False,
 ):
     """Functional API to apply an AdamW optimization step: ``adam`` with decoupled weight decay
     (optimi/adamw.py:78-143)."""
     adam(params, grads, exp_avgs, exp_avg_sqs, kahan_comps, lr=lr, beta1=beta1, beta2=beta2, weight_decay=weight_decay,
          eps=eps, step=step, decouple_wd=True, decouple_lr=decouple_lr, max_lr=max_lr, kahan_sum=kahan_sum,
          foreach=foreach, triton=triton, gradient_release=gradient_release,
-         optimizer_accumulation=optimizer_accumulation, _groups=_groups, _cold=_cold)
+         optimizer_accumulation=optimizer_accumulation, _groups=_groups, _resident=_resident)
 
 
 # --------------------------------------------------------------------------------------
@@ -237,7 +237,7 @@ def lion(
     gradient_release: bool = False,
     optimizer_accumulation: bool = False,
     _groups=None,
-    _cold=False,
+    _resident=False,
 ):
     """Functional API to apply a Lion optimization step (optimi/lion.py:187-266)."""
     _require_hip_backend(triton, foreach, gradient_release)
@@ -249,7 +249,7 @@ def lion(
             weight_decay = 1 - (lr / max_lr) * weight_decay
         else:
             weight_decay = 1 - lr * weight_decay
-    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, COLD=_cold)
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, RESIDENT=_resident)
     scalars = (lr, 1 - beta1, 1 - beta2, weight_decay, flags)
 
     if gradient_release:
@@ -288,7 +288,7 @@ def stableadamw(
     optimizer_accumulation: bool = False,
     mean_squares: list[Tensor] | None = None,
     _groups=None,
-    _cold=False,
+    _resident=False,
 ):
     """Functional API to apply a StableAdamW optimization step (optimi/stableadamw.py:277-371).
 
@@ -306,7 +306,7 @@ def stableadamw(
     t = _tick(step)
     beta1_hat = debias_beta(beta1, t)
     beta2_hat = debias_beta(beta2, t)
-    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, COLD=_cold, DECOUPLE_LR=decouple_lr)
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, RESIDENT=_resident, DECOUPLE_LR=decouple_lr)
     scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps,
                float(max_lr) if (decouple_lr and max_lr is not None) else 0.0, flags)
 
@@ -349,7 +349,7 @@ def adan(
     gradient_release: bool = False,
     optimizer_accumulation: bool = False,
     _groups=None,
-    _cold=False,
+    _resident=False,
 ):
     """Functional API to apply an Adan optimization step (optimi/adan.py:236-350)."""
     _require_hip_backend(triton, foreach, gradient_release)
@@ -364,7 +364,7 @@ def adan(
     if weight_decay != 0:
         weight_decay = (lr / max_lr) * weight_decay if decouple_lr else lr * weight_decay
         weight_decay = 1 - weight_decay if adam_wd else 1 + weight_decay
-    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, COLD=_cold, ADAM_WD=adam_wd)
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, RESIDENT=_resident, ADAM_WD=adam_wd)
     scalars = (lr, 1 - beta1_hat, beta2, 1 - beta2_hat, beta3_hat, 1 - beta3_hat, eps, weight_decay, flags)
 
     if gradient_release:
@@ -400,7 +400,7 @@ def sgd(
     gradient_release: bool = False,
     optimizer_accumulation: bool = False,
     _groups=None,
-    _cold=False,
+    _resident=False,
 ):
     """Functional API to apply a SGD or SGDW optimization step (optimi/sgd.py:213-298)."""
     _require_hip_backend(triton, foreach, gradient_release)
@@ -416,7 +416,7 @@ def sgd(
             weight_decay = 1 - (lr / max_lr) * weight_decay
         elif decouple_wd:
             weight_decay = 1 - lr * weight_decay
-    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, COLD=_cold,
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, RESIDENT=_resident,
                    DECOUPLE_WD=decouple_wd or decouple_lr, DAMPENING=dampening)
     scalars = (lr, momentum, weight_decay, flags)
 
@@ -468,7 +468,7 @@ def radam(
     gradient_release: bool = False,
     optimizer_accumulation: bool = False,
     _groups=None,
-    _cold=False,
+    _resident=False,
 ):
     """Functional API to apply an RAdam optimization step (optimi/radam.py:214-322)."""
     _require_hip_backend(triton, foreach, gradient_release)
@@ -484,7 +484,7 @@ def radam(
             weight_decay = 1 - (lr / max_lr) * weight_decay
         elif decouple_wd:
             weight_decay = 1 - lr * weight_decay
-    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, COLD=_cold,
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, RESIDENT=_resident,
                    DECOUPLE_WD=decouple_wd or decouple_lr, RECTIFY=rect is not None)
     scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps, rect if rect is not None else 0.0, flags)
 
@@ -523,7 +523,7 @@ def ranger(
     gradient_release: bool = False,
     optimizer_accumulation: bool = False,
     _groups=None,
-    _cold=False,
+    _resident=False,
 ):
     """Functional API to apply a Ranger optimization step: RAdam plus Lookahead every ``k`` steps
     (optimi/ranger.py:230-344)."""
@@ -541,7 +541,7 @@ def ranger(
             weight_decay = 1 - (lr / max_lr) * weight_decay
         elif decouple_wd:
             weight_decay = 1 - lr * weight_decay
-    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, COLD=_cold,
+    flags = _flags(ext, kahan_sum=kahan_sum, update_parameters=not optimizer_accumulation, RESIDENT=_resident,
                    DECOUPLE_WD=decouple_wd or decouple_lr, RECTIFY=rect is not None, LOOKAHEAD=t % k == 0)
     scalars = (lr, 1 - beta1_hat, beta2_hat, 1 - beta2_hat, weight_decay, eps, rect if rect is not None else 0.0, alpha, flags)
 

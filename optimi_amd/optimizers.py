@@ -62,11 +62,13 @@ class OptimiOptimizer(Optimizer):
     # that up to _QUEUE_MAX_BYTES of gradients (plus one tensor) stay alive until their launch.
     # Set on the instance, or on the class, before prepare_for_gradient_release.
     native_step = True                      # False: walk the parameters in Python on every step (same results)
-    # How a whole-group step reads its tensors.  None: decided from the optimizer's size - when all its
-    # parameters, gradients and states together fit the GPU's last-level cache, a step finds them there
-    # from the step before and reads them with cached loads; otherwise every list, also the few norm
-    # weights of a small group, is streamed.  True / False force the one or the other.  Results are the same.
-    resident_lists: bool | None = None
+    # How a whole-group step reads its tensors.  False: with streaming loads - right for training, where a
+    # forward and a backward pass run between two steps and nothing of the optimizer's tensors is left in
+    # the GPU's last-level cache.  True: the caller steps back to back with nothing in between (a benchmark
+    # loop); if the optimizer's parameters, gradients and states together fit that cache, a step finds them
+    # there and reads them with cached loads, 1 % faster then and 8 % slower if the cache was swept after
+    # all.  Results are the same either way.
+    resident_lists: bool = False
     gradient_release_coalesce = 1 << 26
     _QUEUE_MAX_TENSORS = 1024               # parked steps per launch
     _QUEUE_MAX_BYTES = 128 << 20            # bytes of parked gradients kept alive at most
@@ -107,7 +109,7 @@ class OptimiOptimizer(Optimizer):
         self._hip_groups: dict = {}
         self._release_queue = None
         self._release_hook = None
-        self._cold = None
+        self._fits_cache = None
 
         if self.defaults["gradient_release"]:
             if self.defaults["foreach"]:  # optimi/optimizer.py:65-68
@@ -126,7 +128,7 @@ class OptimiOptimizer(Optimizer):
         state.pop("_hip_groups", None)
         state.pop("_release_queue", None)
         state.pop("_release_hook", None)
-        state.pop("_cold", None)
+        state.pop("_fits_cache", None)
         return state
 
     def __setstate__(self, state):
@@ -134,7 +136,7 @@ class OptimiOptimizer(Optimizer):
         self.__dict__.setdefault("_hip_groups", {})
         self.__dict__.setdefault("_release_queue", None)
         self.__dict__.setdefault("_release_hook", None)
-        self.__dict__["_cold"] = None
+        self.__dict__["_fits_cache"] = None
         self._invalidate_release_cache()
         self.__dict__.setdefault("_optimizer_accumulation", False)
 
@@ -238,10 +240,10 @@ class OptimiOptimizer(Optimizer):
         if param is None:
             self._flush_release()
             driver = self._driver() if self.native_step else None
-            cold = self._lists_are_cold()
+            resident = self._lists_are_resident()
             for group in self.param_groups:
                 # after a group's first step the whole walk over its parameters is native
-                if driver is not None and group["setup"] and driver.step_group(group, cold):
+                if driver is not None and group["setup"] and driver.step_group(group, resident):
                     continue
                 params = self._collect(group)
                 if params and not group["triton"]:
@@ -348,24 +350,25 @@ class OptimiOptimizer(Optimizer):
         return backend.ext().ReleaseHook(self._driver())
 
     def _invalidate_release_cache(self):
-        self.__dict__["_cold"] = None
+        self.__dict__["_fits_cache"] = None
         self.__dict__.get("_hip_groups", {}).clear()  # keyed by group dicts that may be gone now
         if self.__dict__.get("_release_hook") is not None:
             self._release_hook.invalidate()
 
-    def _lists_are_cold(self) -> bool:
-        """Whether a whole-group step must take its tensors for gone from the last-level cache since the
-        previous step: they are when everything the optimizer touches in a step is larger than that cache."""
-        if self.resident_lists is not None:
-            return not self.resident_lists
-        if self._cold is None:
+    def _lists_are_resident(self) -> bool:
+        """Whether a whole-group step may take its tensors for still being in the last-level cache from
+        the step before: the caller has said that it steps back to back (``resident_lists``), and
+        everything the optimizer touches in a step - all groups together - fits that cache."""
+        if not self.resident_lists:
+            return False
+        if self._fits_cache is None:
             total = 0
             for group in self.param_groups:
                 for p in group["params"]:
                     arrays = 2 + len(self._moment_keys) + (1 if p.dtype in _LOW_PRECISION else 0)
                     total += p.numel() * p.element_size() * arrays
-            self._cold = total > backend.ext().resident_bytes()
-        return self._cold
+            self._fits_cache = total <= backend.ext().resident_bytes()
+        return self._fits_cache
 
     def _workspaces(self, group: dict) -> dict:
         """The launch workspaces of one parameter group: its device tables then keep this group's list
@@ -466,7 +469,7 @@ class Adam(OptimiOptimizer):
                lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"], weight_decay=group["weight_decay"],
                eps=group["eps"], step=step, decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"],
                max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
-               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
+               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._workspaces(group), _resident=self._lists_are_resident())
 
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
@@ -544,7 +547,7 @@ class Lion(OptimiOptimizer):
         F.lion(params, grads, _col(states, "exp_avg"), _col(states, "kahan_comp"), lr=group["lr"], beta1=group["beta1"],
                beta2=group["beta2"], weight_decay=group["weight_decay"], decouple_lr=group["decouple_lr"],
                max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
-               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
+               gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._workspaces(group), _resident=self._lists_are_resident())
 
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
@@ -619,7 +622,7 @@ class StableAdamW(OptimiOptimizer):
                       weight_decay=group["weight_decay"], eps=group["eps"], step=step, decouple_lr=group["decouple_lr"],
                       max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
                       gradient_release=gradient_release, optimizer_accumulation=accumulate, mean_squares=None,
-                      _groups=self._workspaces(group), _cold=self._lists_are_cold())
+                      _groups=self._workspaces(group), _resident=self._lists_are_resident())
 
 
     def _release_workspace(self, param):
@@ -694,7 +697,7 @@ class Adan(OptimiOptimizer):
                beta2=group["beta2"], beta3=group["beta3"], eps=group["eps"], weight_decay=group["weight_decay"],
                step=step, decouple_lr=group["decouple_lr"], max_lr=group["max_lr"], kahan_sum=group["kahan_sum"],
                foreach=False, triton=True, gradient_release=gradient_release,
-               optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
+               optimizer_accumulation=accumulate, _groups=self._workspaces(group), _resident=self._lists_are_resident())
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
         # adam_wd is not forwarded, as in step() above
@@ -776,7 +779,7 @@ class SGD(OptimiOptimizer):
               momentum=group["momentum"], weight_decay=group["weight_decay"], dampening=group["dampening"],
               decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"], max_lr=group["max_lr"],
               kahan_sum=group["kahan_sum"], foreach=False, triton=True, gradient_release=gradient_release,
-              optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
+              optimizer_accumulation=accumulate, _groups=self._workspaces(group), _resident=self._lists_are_resident())
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
         return ext.sgd_release(param, grad, state["exp_avg"], state["kahan_comp"], group["lr"], group["momentum"],
@@ -830,7 +833,7 @@ class RAdam(OptimiOptimizer):
                 lr=group["lr"], beta1=group["beta1"], beta2=group["beta2"], weight_decay=group["weight_decay"],
                 eps=group["eps"], step=step, decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"],
                 max_lr=group["max_lr"], kahan_sum=group["kahan_sum"], foreach=False, triton=True,
-                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
+                gradient_release=gradient_release, optimizer_accumulation=accumulate, _groups=self._workspaces(group), _resident=self._lists_are_resident())
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
         return ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], None, state["kahan_comp"], state["step"],
@@ -892,7 +895,7 @@ class Ranger(OptimiOptimizer):
                  weight_decay=group["weight_decay"], eps=group["eps"], k=group["k"], alpha=group["alpha"], step=step,
                  decouple_wd=group["decouple_wd"], decouple_lr=group["decouple_lr"], max_lr=group["max_lr"],
                  kahan_sum=group["kahan_sum"], foreach=False, triton=True, gradient_release=gradient_release,
-                 optimizer_accumulation=accumulate, _groups=self._workspaces(group), _cold=self._lists_are_cold())
+                 optimizer_accumulation=accumulate, _groups=self._workspaces(group), _resident=self._lists_are_resident())
 
     def _release_call(self, ext, group, state, param, grad, update, queue):
         return ext.ranger_release(param, grad, state["exp_avg"], state["exp_avg_sq"], state["la_param"], state["kahan_comp"],

@@ -28,10 +28,10 @@ class HipRun(ForLoopRun):
     A list whose tensors differ in dtype goes through the ``_multi_mixed`` entry points;
     ``mixed=True`` sends a list of one dtype through them as well."""
 
-    def __init__(self, name, params, *, multi=True, cold=False, mixed=False, **kw):
+    def __init__(self, name, params, *, multi=True, resident=False, mixed=False, **kw):
         super().__init__(name, params, **kw)
         self.multi = multi
-        self.cold = cold  # pass OPTIMI_COLD to the whole-list entry points
+        self.resident = resident  # pass OPTIMI_RESIDENT to the whole-list entry points
         self.mixed = mixed
         self.group = cabi.Group()
         self.entry = "adam" if name == "adamw" else name
@@ -70,8 +70,8 @@ class HipRun(ForLoopRun):
             return
         dt = DT[ps[0].dtype]
         if self.multi and not self.gradient_release:
-            if self.cold:
-                scalars = scalars[:-1] + (scalars[-1] | cabi.COLD,)
+            if self.resident:
+                scalars = scalars[:-1] + (scalars[-1] | cabi.RESIDENT,)
             cols = [cabi.ptr_array(_addr(p) for p in ps), cabi.ptr_array(_addr(g) for g in grads)]
             cols += [cabi.ptr_array(_addr(s[k]) for s in sts) for k in STATE_ORDER[self.name]]
             cols.append(cabi.ptr_array(_addr(s["kahan_comp"]) for s in sts))

@@ -39,7 +39,7 @@ def test_error_strings_and_constants():
     # the flag values the Python side uses are the header's
     text = open(HEADER).read()
     for name, val in (("KAHAN", cabi.KAHAN), ("UPDATE", cabi.UPDATE), ("DECOUPLE_WD", cabi.DECOUPLE_WD),
-                      ("ADAM_WD", cabi.ADAM_WD), ("DECOUPLE_LR", cabi.DECOUPLE_LR), ("COLD", cabi.COLD),
+                      ("ADAM_WD", cabi.ADAM_WD), ("DECOUPLE_LR", cabi.DECOUPLE_LR), ("RESIDENT", cabi.RESIDENT),
                       ("PROBE_SCRAMBLE", cabi.PROBE_SCRAMBLE)):
         assert re.search(rf"OPTIMI_{name}\s*=\s*{val}\b", text), name
 

@@ -83,10 +83,11 @@ def test_load_state_dict_and_add_param_group_drop_the_cached_tables(hip_device):
     torch.cuda.synchronize()
 
 
-def test_cached_or_streaming_loads_are_decided_for_the_whole_optimizer(hip_device):
-    """A small model lives in the last-level cache and is read with cached loads.  The same small group
-    beside a group that does not fit the cache is cold every time it is stepped, and must be streamed -
-    as must everything when the caller says so.  (Bits never depend on this: see test_cold_hint_changes_nothing.)"""
+def test_cached_loads_are_opt_in_and_decided_for_the_whole_optimizer(hip_device):
+    """By default every list is streamed (a training loop sweeps the cache between steps).  With
+    ``resident_lists = True`` a small model is read with cached loads - but the same small group beside a
+    group that does not fit the cache is cold every time it is stepped, and stays streamed.  Both
+    walks agree.  (Bits never depend on this: see test_resident_hint_changes_nothing.)"""
     L = cabi.lib()
     ext = optimi_amd.backend.ext()
     limit = ext.resident_bytes()
@@ -95,29 +96,30 @@ def test_cached_or_streaming_loads_are_decided_for_the_whole_optimizer(hip_devic
     def resident_launches(opt, params):
         for p in params:
             p.grad = torch.full_like(p, 1e-3)
-        opt.step()  # the first step of a group is set up in Python; both walks must agree, so count over two steps
+        opt.step()  # the first step of a group is set up in Python; count a later one
         before = L.optimi_hip_resident_launch_count()
         opt.step()
         return L.optimi_hip_resident_launch_count() - before
 
     mats, vecs = two_groups(hip_device, seed=5)
     small = optimi_amd.AdamW([{"params": mats}, {"params": vecs, "weight_decay": 0.0}], lr=1e-3)
-    assert not small._lists_are_cold()
+    assert not small._lists_are_resident()
+    assert resident_launches(small, mats + vecs) == 0
+    small.resident_lists = True
+    assert small._lists_are_resident()
+    assert resident_launches(small, mats + vecs) == 2
+    small.native_step = False
     assert resident_launches(small, mats + vecs) == 2
     small.resident_lists = False
     assert resident_launches(small, mats + vecs) == 0
-    small.resident_lists = None
-    small.native_step = False
-    assert resident_launches(small, mats + vecs) == 2
 
     # one bf16 tensor whose five arrays (parameter, gradient, two moments, Kahan buffer) exceed the limit
     big = torch.nn.Parameter(torch.zeros(limit // 10 + 4096, dtype=torch.bfloat16, device=hip_device))
     mats2, vecs2 = two_groups(hip_device, seed=6)
     large = optimi_amd.AdamW([{"params": [big] + mats2}, {"params": vecs2, "weight_decay": 0.0}], lr=1e-3)
-    assert large._lists_are_cold()
+    large.resident_lists = True
+    assert not large._lists_are_resident()  # the hint is given, the optimizer as a whole does not fit
     assert resident_launches(large, [big] + mats2 + vecs2) == 0
     large.native_step = False
     assert resident_launches(large, [big] + mats2 + vecs2) == 0
-    large.resident_lists = True
-    assert resident_launches(large, [big] + mats2 + vecs2) == 1  # the small group; the big one is over the limit on its own
     torch.cuda.synchronize()

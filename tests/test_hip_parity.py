@@ -259,21 +259,21 @@ def test_list_lengths_around_the_kernel_argument_table(cfg, n_tensors, hip_devic
 
 @pytest.mark.parametrize("cfg", ["adamw", "lion", "stableadamw", "adan", "sgd_momentum", "ranger"])
 @pytest.mark.parametrize("n_tensors", [5, 19])
-def test_cold_hint_changes_nothing(cfg, n_tensors, hip_device):
-    """A small list is read with cached loads, the same list marked OPTIMI_COLD with streaming
+def test_resident_hint_changes_nothing(cfg, n_tensors, hip_device):
+    """A small list is read with streaming loads, the same list marked OPTIMI_RESIDENT with cached
     loads: two copies of the tile body in the kernel, one set of bits."""
     from hip_engine import HipRun
 
     hyper, name = CONFIGS[cfg], OPT_OF[cfg]
     sizes = SIZES[-n_tensors:]
     params, grads = draw(sizes, torch.bfloat16, 4, seed=31)
-    warm = HipRun(name, [p.to(hip_device) for p in params], **hyper)
-    cold = HipRun(name, [p.to(hip_device) for p in params], cold=True, **hyper)
+    warm = HipRun(name, [p.to(hip_device) for p in params], resident=True, **hyper)
+    cold = HipRun(name, [p.to(hip_device) for p in params], **hyper)
     for gs in grads:
         warm.step([g.to(hip_device) for g in gs])
         cold.step([g.to(hip_device) for g in gs])
     torch.cuda.synchronize()
-    G.compare_engines(cold, warm, f"{cfg} cold vs resident", exact=True)
+    G.compare_engines(cold, warm, f"{cfg} streaming vs cached loads", exact=True)
 
 
 def test_rejected_arguments_on_device(hip_device):

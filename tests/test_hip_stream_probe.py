@@ -45,7 +45,7 @@ def test_probe_touches_what_it_says(hip_device, n_read, n_write, n_tensors):
     table, keep = cabi.ptr_table([[v.data_ptr() if v.numel() else None for v in col] for col in views])
     group = cabi.Group()
     stream = torch.cuda.current_stream().cuda_stream
-    for granules, flags in ((0, 0), (9, cabi.PROBE_SCRAMBLE), (0, cabi.PROBE_SCRAMBLE | cabi.COLD), (14, 0)):
+    for granules, flags in ((0, 0), (9, cabi.PROBE_SCRAMBLE), (0, cabi.PROBE_SCRAMBLE | cabi.RESIDENT), (14, 0)):
         before = [[v.clone() for v in col] for col in views]
         launches = L.optimi_hip_launch_count()
         cabi.check(L.optimi_hip_stream_probe(group.handle, n_tensors, table, cabi.i64_array(sizes), n_read, n_write, granules,
