@@ -74,12 +74,21 @@ def workloads():
         # the same list with the embeddings and the norm weights kept in fp32 (FP32_TENSORS): one launch over both
         # dtypes; 18 bytes per bf16 parameter, 28 per fp32 one
         "adamw_bf16_kahan_fp32_embeddings_norms_llama7b": ("AdamW", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2), "bfloat16", l7, 18),
+        # the same list as two parameter groups, as param_groups_weight_decay makes them: the 226 matrices decay, the 64
+        # norm weights do not (TWO_GROUPS) - two launches per step, each group with its own device tables
+        "adamw_bf16_kahan_decay_nodecay_llama7b": ("AdamW", dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2), "bfloat16", l7, 18),
     }
 
 
 # workload -> which tensors of its list are fp32 instead of the workload's dtype
 FP32_TENSORS = {
     "adamw_bf16_kahan_fp32_embeddings_norms_llama7b": lambda shape: len(shape) == 1 or shape[0] == 32000,
+}
+
+
+# workload -> which tensors of its list go into a second parameter group without weight decay
+TWO_GROUPS = {
+    "adamw_bf16_kahan_decay_nodecay_llama7b": lambda shape: len(shape) == 1,
 }
 
 
@@ -101,7 +110,8 @@ MEASURED_TRAFFIC = {
 # the benchmark configurations reported under "extra" next to the headline workload
 EXTRA_WORKLOADS = [
     "adamw_fp32_mlp", "adamw_bf16_kahan_declr_llama1b", "lion_bf16_kahan_llama7b", "stableadamw_bf16_kahan_llama7b",
-    "adan_bf16_kahan_llama7b", "adamw_bf16_kahan_fp32_embeddings_norms_llama7b", "adamw_bf16_kahan_release_llama7b",
+    "adan_bf16_kahan_llama7b", "adamw_bf16_kahan_fp32_embeddings_norms_llama7b", "adamw_bf16_kahan_decay_nodecay_llama7b",
+    "adamw_bf16_kahan_release_llama7b",
     "adamw_bf16_kahan_release_stress10k",
 ]
 RELEASE_WORKLOADS = ("adamw_bf16_kahan_release_stress10k", "adamw_bf16_kahan_release_llama7b")
@@ -429,7 +439,13 @@ def list_bench(workload, args, steps, warmup):
     misalign = getattr(args, "misalign", 0)
     params = [torch.nn.Parameter(p) for p in make_tensors(shapes, dtypes, device, 0, 0.02, ones_for_1d=True, misalign=misalign)]
     grad_sets = [make_tensors(shapes, dtypes, device, 100 + i, 1e-3, misalign=misalign) for i in range(max(1, args.grad_sets))]
-    opt = getattr(optimi_amd, cls_name)(params, **kwargs)
+    no_decay = TWO_GROUPS.get(workload)
+    if no_decay:
+        groups = [{"params": [p for p, s in zip(params, shapes) if not no_decay(s)]},
+                  {"params": [p for p, s in zip(params, shapes) if no_decay(s)], "weight_decay": 0.0}]
+        opt = getattr(optimi_amd, cls_name)(groups, **kwargs)
+    else:
+        opt = getattr(optimi_amd, cls_name)(params, **kwargs)
 
     def one_step(i):
         for p, g in zip(params, grad_sets[i % len(grad_sets)]):
@@ -493,6 +509,7 @@ def list_bench(workload, args, steps, warmup):
         "data": "synthetic",
         "config": {"workload": workload, "optimizer": cls_name, "n_tensors": len(shapes), "n_params": n_params,
                    **({"n_params_fp32": n_fp32} if is_fp32 else {}), **({"misalign_elements": misalign} if misalign else {}),
+                   **({"param_groups": [len(g["params"]) for g in opt.param_groups]} if no_decay else {}),
                    "hyper": {k: (list(v) if isinstance(v, tuple) else v) for k, v in kwargs.items()},
                    "grad_sets": len(grad_sets)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
