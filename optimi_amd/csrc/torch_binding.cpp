@@ -1099,12 +1099,17 @@ class ReleaseHookCore {
     }
     return v;
   }
+  // Values that can change without the dict that holds them changing (a tensor learning rate
+  // filled in place, a user's own number type) must be read afresh on every call.
+  static inline thread_local bool read_only_immutables_ = true;
   static double as_double(PyObject* v) {
+    if (!PyFloat_CheckExact(v) && !PyLong_CheckExact(v)) read_only_immutables_ = false;
     const double d = PyFloat_AsDouble(v);
     if (d == -1.0 && PyErr_Occurred()) throw py::error_already_set();
     return d;
   }
   static bool truthy(PyObject* v) {
+    if (v != Py_True && v != Py_False && v != Py_None) read_only_immutables_ = false;
     const int r = PyObject_IsTrue(v);
     if (r < 0) throw py::error_already_set();
     return r == 1;
@@ -1149,10 +1154,11 @@ class ReleaseHookCore {
     }
     if (version == 0 || slot->version != version || slot->t != t || slot->update != update) {
       slot->version = 0;  // void while it is being rebuilt (read_hyper may throw)
+      read_only_immutables_ = true;
       slot->h = read_hyper(grp, t, update);
       slot->t = t;
       slot->update = update;
-      slot->version = version;
+      slot->version = read_only_immutables_ ? version : 0;  // 0: read again next time
     }
     return slot->h;
   }

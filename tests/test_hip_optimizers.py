@@ -789,3 +789,44 @@ def test_two_optimizers_stepping_from_two_threads(hip_device):
     assert not errors, errors
     for name, (opt, params, ref) in results.items():
         compare(opt, params, ref, f"threaded {name}")
+
+
+@pytest.mark.parametrize("release", [False, True], ids=["step", "gradient_release"])
+def test_a_tensor_learning_rate_filled_in_place_is_seen(release, hip_device):
+    """torch's schedulers fill a tensor learning rate in place (``param_group["lr"].fill_(x)``): the group
+    dict is not modified then, so the native drivers, which reuse a group's step scalars while its dict is
+    unmodified, must not reuse them for values that can change underneath it.  An optimizer whose lr is a
+    float64 tensor, filled in place between steps, against one that is handed plain floats."""
+    gen = torch.Generator().manual_seed(41)
+    shapes = [(40, 30), (8200,), (64,)] * 6
+    start = [(torch.randn(s, generator=gen) * 0.02).to(torch.bfloat16).to(hip_device) for s in shapes]
+    models = []
+    for lr in (torch.tensor(1e-3, dtype=torch.float64), 1e-3):
+        model = torch.nn.Module()
+        model.ps = torch.nn.ParameterList([torch.nn.Parameter(p.clone()) for p in start])
+        opt = optimi_amd.AdamW(model.parameters(), lr=lr, weight_decay=1e-2, gradient_release=release)
+        if release:
+            optimi_amd.prepare_for_gradient_release(model, opt)
+        models.append((model, opt))
+    lrs = [1e-3, 1e-3, 5e-4, 5e-4, 2.5e-4, 1e-3]
+    for it, lr in enumerate(lrs):
+        models[0][1].param_groups[0]["lr"].fill_(lr)   # in place: the dict keeps the same tensor object
+        models[1][1].param_groups[0]["lr"] = lr
+        grads = [(torch.randn(s, generator=gen) * 1e-3).to(torch.bfloat16).to(hip_device) for s in shapes]
+        for model, opt in models:
+            if release:
+                loss = sum((p * g).sum() for p, g in zip(model.ps, grads))
+                loss.backward()
+            else:
+                for p, g in zip(model.ps, grads):
+                    p.grad = g.clone()
+                opt.step()
+                opt.zero_grad()
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(zip(models[0][0].ps, models[1][0].ps)):
+        G.assert_bits_equal(a, b, f"param {i}")
+        for key in ("exp_avg", "exp_avg_sq", "kahan_comp"):
+            G.assert_bits_equal(models[0][1].state[a][key], models[1][1].state[b][key], f"{key} {i}")
+    for model, _ in models:
+        if release:
+            optimi_amd.remove_gradient_release(model)
