@@ -687,8 +687,11 @@ def main():
                 continue
             # short launches are timed over more steps: a 0.1 ms step needs many to average the host's jitter out
             steps = 200 if name == "adamw_fp32_mlp" else (40 if "llama1b" in name else (16 if name in RELEASE_WORKLOADS else 12))
-            line, _ = run_workload(name, args, steps, 8 if name in RELEASE_WORKLOADS else 5)
+            line, extra_spec = run_workload(name, args, steps, 8 if name in RELEASE_WORKLOADS else 5)
             extra[name] = brief(line)
+            if name == "adamw_fp32_mlp" and extra_spec is not None and not args.no_cpu_baseline:
+                # benchmark configuration 1 is the reference's own CPU-runnable case: the whole list, a few seconds
+                extra[name]["cpu_baseline"] = cpu_baseline(*extra_spec, budget_s=6.0)
             gc.collect()
         extra["adamw_fp32_mlp_cold"] = cold_cache_bench(args)
         gc.collect()
