@@ -113,6 +113,10 @@ EXTRA_WORKLOADS = [
     "adan_bf16_kahan_llama7b", "adamw_bf16_kahan_fp32_embeddings_norms_llama7b", "adamw_bf16_kahan_decay_nodecay_llama7b",
     "adamw_bf16_kahan_release_llama7b",
     "adamw_bf16_kahan_release_stress10k",
+    # the optimizers and dtypes beyond the benchmark configurations, so that every figure quoted anywhere is timed by
+    # whoever runs this file
+    "sgd_bf16_kahan_llama7b", "radam_bf16_kahan_llama7b", "ranger_bf16_kahan_llama7b", "adamw_fp16_kahan_llama7b",
+    "adamw_fp32_llama1b",
 ]
 RELEASE_WORKLOADS = ("adamw_bf16_kahan_release_stress10k", "adamw_bf16_kahan_release_llama7b")
 
