@@ -179,10 +179,19 @@ def test_headline_adamw_llama7b_whole_list_against_emulator(hip_device):
     params = draw(shapes, hip_device, gen, 0.02, ones_for_1d=True)
     hip = HipRun("adamw", params, **ADAMW)
     sca = ScalarRun("adamw", [p.cpu() for p in params], **ADAMW)
+    # the gradients travel to the host through one pinned buffer (13.5 GB): a pageable copy of each tensor is five times slower
+    stage = torch.empty(sum(math.prod(s) for s in shapes), dtype=torch.bfloat16, pin_memory=True)
+    offsets = [0]
+    for s in shapes:
+        offsets.append(offsets[-1] + math.prod(s))
+    host_grads = [stage[a:b].view(s) for a, b, s in zip(offsets, offsets[1:], shapes)]
     for _ in range(10):
         grads = draw(shapes, hip_device, gen, 1e-3)
         hip.step(grads)
-        sca.step([g.cpu() for g in grads])
+        for h, g in zip(host_grads, grads):
+            h.copy_(g, non_blocking=True)
+        torch.cuda.synchronize()
+        sca.step(host_grads)  # the emulator reads the gradients and leaves them as they are
         del grads
     torch.cuda.synchronize()
     # compared on the device, tensor by tensor: the oracle's result travels up, 5 x 13.5 GB in all
