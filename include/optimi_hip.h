@@ -64,7 +64,7 @@ enum optimi_flags {
 enum optimi_status {
   OPTIMI_OK = 0,
   OPTIMI_ERR_NULL = -1,      /* a required pointer is NULL                         */
-  OPTIMI_ERR_SIZE = -2,      /* negative element or tensor count                   */
+  OPTIMI_ERR_SIZE = -2,      /* negative element or tensor count, or beyond limits */
   OPTIMI_ERR_DTYPE = -3,     /* dtype is not an optimi_dtype                       */
   OPTIMI_ERR_ALIGN = -4,     /* a buffer is not aligned to its element size        */
   OPTIMI_ERR_DEVICE = -5,    /* group used on a device other than the one it was made on */
@@ -322,6 +322,16 @@ int64_t optimi_hip_resident_bytes(void);
  * how many of the kernels launched for lists read their tensors with cached loads. */
 int64_t optimi_hip_upload_count(void);
 int64_t optimi_hip_resident_launch_count(void);
+
+/* Test aid (no counterpart in the reference).  A HIP grid holds fewer than 2^32 threads, i.e.
+ * fewer than 2^26 of this library's 64-lane workgroups, which is 64 GiB per array; a longer list
+ * or tensor (up to 2^31 / 16 chunks of 16 KiB per array, and 2^24 - 1 tensors: OPTIMI_ERR_SIZE
+ * beyond) is stepped by several launches, each starting where the previous one ended.  This call
+ * sets the number of workgroups one launch may hold - rounded down to whole chunks (16
+ * workgroups), at least one chunk, at most the hardware's limit - so that tests can run the
+ * split on small lists; 0 changes nothing, a negative value restores the hardware's limit.
+ * Returns the limit that was in force before.  Results never depend on it. */
+int64_t optimi_hip_launch_limit(int64_t workgroups);
 
 #ifdef __cplusplus
 }

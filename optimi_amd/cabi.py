@@ -55,6 +55,7 @@ PROTOTYPES = {
     "optimi_hip_resident_bytes": (_i64, []),
     "optimi_hip_upload_count": (_i64, []),
     "optimi_hip_resident_launch_count": (_i64, []),
+    "optimi_hip_launch_limit": (_i64, [_i64]),
 }
 
 _lib = None

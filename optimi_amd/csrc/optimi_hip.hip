@@ -60,7 +60,7 @@ constexpr int kSub = kChunkBytes / (kThreads * kUnroll * 16);  // workgroups per
 static_assert(kSub >= 1 && kSub * kThreads * kUnroll * 16 == kChunkBytes, "workgroup tile must divide the chunk");
 static_assert(kThreads % 64 == 0 && kThreads <= 1024, "whole wavefronts");
 constexpr int kReduceThreads = 1024;      // lanes of the per-tensor finalize workgroup
-constexpr int kAbiVersion = 1003;
+constexpr int kAbiVersion = 1004;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -768,7 +768,7 @@ __device__ __forceinline__ void tile_step(const TensorEntry& e, int tensor, int6
   if (Op::kReduce) {
     __shared__ double lds[kThreads / 64];
     double total = block_sum<kThreads>((double)acc, lds);
-    if (threadIdx.x == 0) partials[blockIdx.x] = total;
+    if (threadIdx.x == 0) partials[chunk_id * kSub + sub] = total;
   }
 }
 
@@ -778,9 +778,11 @@ __device__ __forceinline__ void tile_step(const TensorEntry& e, int tensor, int6
 template <class Op, bool MULTI>
 __global__ void __launch_bounds__(kThreads)
 step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, const FewTable few,
-            typename Op::Scalars s, double* __restrict__ partials) {
-  const int64_t chunk_id = blockIdx.x / kSub;
-  const int sub = blockIdx.x % kSub;
+            typename Op::Scalars s, double* __restrict__ partials, int64_t first_workgroup) {
+  // a list too long for one grid is stepped by several launches; this one starts at `first_workgroup`
+  const int64_t workgroup = first_workgroup + blockIdx.x;
+  const int64_t chunk_id = workgroup / kSub;
+  const int sub = (int)(workgroup % kSub);
   // a table of one (the per-tensor entry points) needs no search
   const int tensor = MULTI ? chunk_map[chunk_id] : (few.n == 1 ? 0 : optimi_tables::few_lookup(few, chunk_id));
   const TensorEntry& e = MULTI ? table[tensor] : few.e[tensor];
@@ -794,9 +796,11 @@ step_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ c
 template <class OpLow, class OpF32, bool MULTI>
 __global__ void __launch_bounds__(kThreads)
 mixed_kernel(const TensorEntry* __restrict__ table, const int32_t* __restrict__ chunk_map, const FewTable few,
-             typename OpLow::Scalars s_low, typename OpF32::Scalars s_f32, double* __restrict__ partials) {
-  const int64_t chunk_id = blockIdx.x / kSub;
-  const int sub = blockIdx.x % kSub;
+             typename OpLow::Scalars s_low, typename OpF32::Scalars s_f32, double* __restrict__ partials,
+             int64_t first_workgroup) {
+  const int64_t workgroup = first_workgroup + blockIdx.x;
+  const int64_t chunk_id = workgroup / kSub;
+  const int sub = (int)(workgroup % kSub);
   const int tensor = MULTI ? chunk_map[chunk_id] : optimi_tables::few_lookup(few, chunk_id);
   const TensorEntry& e = MULTI ? table[tensor] : few.e[tensor];
   if (e.flags & optimi_tables::kEntryF32) tile_step<OpF32>(e, tensor, chunk_id, sub, s_f32, partials);
@@ -1014,7 +1018,7 @@ struct ListPlan {
   bool misaligned = false;    // most of the list's elements are in tensors with a buffer off the 16-byte grid
 };
 
-constexpr int64_t kMaxChunks = (int64_t)0x7fffffff / kSub;  // the grid is chunks x kSub workgroups
+constexpr int64_t kMaxChunks = (int64_t)0x7fffffff / kSub;  // chunk and workgroup numbers fit 31 bits (2 TiB per array)
 
 // The dtypes a mixed list may hold: fp32 and at most one 16-bit dtype.  `*low` becomes the
 // dtype of the tensors that are not fp32 (fp32 if there are none), `*mixed` whether both kinds
@@ -1271,31 +1275,42 @@ const FewTable kNoTable = {};
 std::atomic<int64_t> kernel_launches{0};  // every kernel this library has launched in this process
 std::atomic<int64_t> resident_launches{0};  // list launches among them that read with cached loads
 
+// A grid holds fewer than 2^32 threads: a launch of 2^26 or more 64-lane workgroups is refused by
+// the runtime when the count is an exact multiple of 2^26 and otherwise runs only the count
+// modulo 2^26 without any error (measured: 2^26 + 16 workgroups ran 16).  Lists beyond that -
+// more than 64 GiB per array - are stepped by several launches of whole chunks, each told where
+// it starts.  The limit is a variable so that tests can exercise the split on small lists.
+constexpr int64_t kGridWorkgroups = ((int64_t)1 << 32) / kThreads - kSub;
+std::atomic<int64_t> launch_workgroup_limit{kGridWorkgroups};
+
 // `s_f32`: the same scalars formed for fp32 tensors; read only when the plan is a mixed list.
 template <class Op>
 void launch_list(optimi_group* g, const ListPlan& plan, const typename Op::Scalars& s, hipStream_t stream,
                  double* partials = nullptr, const typename Op::Scalars* s_f32 = nullptr, int granules = 0) {
   const int64_t workgroups = plan.n_chunks * kSub;
   const LaunchShape shape = launch_shape<Op>(workgroups, plan.few, plan.misaligned, granules);
-  ++kernel_launches;
   if (plan.resident) ++resident_launches;
-  if constexpr (!std::is_same<typename Op::DT, F32>::value) {
-    if (plan.mixed) {
-      if (plan.few)
-        mixed_kernel<Op, typename Op::F32Partner, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
-            nullptr, nullptr, plan.table, s, *s_f32, partials);
-      else
-        mixed_kernel<Op, typename Op::F32Partner, true><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
-            (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, *s_f32, partials);
-      return;
+  const int64_t limit = launch_workgroup_limit.load();
+  for (int64_t first = 0; first < workgroups; first += limit) {
+    const dim3 grid((unsigned)(workgroups - first < limit ? workgroups - first : limit));
+    ++kernel_launches;
+    if constexpr (!std::is_same<typename Op::DT, F32>::value) {
+      if (plan.mixed) {
+        if (plan.few)
+          mixed_kernel<Op, typename Op::F32Partner, false><<<grid, dim3(kThreads), shape.lds, stream>>>(
+              nullptr, nullptr, plan.table, s, *s_f32, partials, first);
+        else
+          mixed_kernel<Op, typename Op::F32Partner, true><<<grid, dim3(kThreads), shape.lds, stream>>>(
+              (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, *s_f32, partials, first);
+        continue;
+      }
     }
+    if (plan.few)
+      step_kernel<Op, false><<<grid, dim3(kThreads), shape.lds, stream>>>(nullptr, nullptr, plan.table, s, partials, first);
+    else
+      step_kernel<Op, true><<<grid, dim3(kThreads), shape.lds, stream>>>(
+          (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, partials, first);
   }
-  if (plan.few)
-    step_kernel<Op, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
-        nullptr, nullptr, plan.table, s, partials);
-  else
-    step_kernel<Op, true><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
-        (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, partials);
 }
 
 inline FewTable table_of_one(const TensorEntry& e) {
@@ -1311,9 +1326,13 @@ void launch_single(const TensorEntry& e, const typename Op::Scalars& s, double* 
   const int64_t chunk = chunk_elems<typename Op::DT>();
   const int64_t workgroups = (e.numel + chunk - 1) / chunk * kSub;
   const LaunchShape shape = launch_shape<Op>(workgroups, true, !(e.flags & optimi_tables::kEntryVec));
-  ++kernel_launches;
-  step_kernel<Op, false><<<dim3((unsigned)workgroups), dim3(kThreads), shape.lds, stream>>>(
-      nullptr, nullptr, table_of_one(e), s, partials);
+  const FewTable one = table_of_one(e);
+  const int64_t limit = launch_workgroup_limit.load();
+  for (int64_t first = 0; first < workgroups; first += limit) {
+    ++kernel_launches;
+    step_kernel<Op, false><<<dim3((unsigned)(workgroups - first < limit ? workgroups - first : limit)), dim3(kThreads), shape.lds,
+                             stream>>>(nullptr, nullptr, one, s, partials, first);
+  }
 }
 
 // Calls fn(Op{}) for the Op selected by dtype x kahan x update x weight-decay mode.  NWD is
@@ -2243,12 +2262,29 @@ int optimi_hip_copy_probe(void* dst, const void* src, int64_t bytes, optimi_stre
   if (((uintptr_t)dst % 16) || ((uintptr_t)src % 16)) return OPTIMI_ERR_ALIGN;
   const int64_t n_vec = bytes / 16;
   if (n_vec == 0) return 0;
-  const int64_t blocks = (n_vec + 255) / 256;
-  if (blocks > 0x7fffffff) return OPTIMI_ERR_SIZE;
-  ++kernel_launches;
-  copy_probe_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream_>>>((u32x4*)dst, (const u32x4*)src, n_vec);
-  HIP_TRY(hipGetLastError());
+  // fewer than 2^32 threads per grid (see launch_workgroup_limit): just under 64 GiB per launch
+  constexpr int64_t kVecPerLaunch = (((int64_t)1 << 32) / 256 - 1) * 256;
+  for (int64_t first = 0; first < n_vec; first += kVecPerLaunch) {
+    const int64_t n = n_vec - first < kVecPerLaunch ? n_vec - first : kVecPerLaunch;
+    ++kernel_launches;
+    copy_probe_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream_>>>((u32x4*)dst + first,
+                                                                                                 (const u32x4*)src + first, n);
+    HIP_TRY(hipGetLastError());
+  }
   return 0;
+}
+
+int64_t optimi_hip_launch_limit(int64_t workgroups) {
+  const int64_t before = launch_workgroup_limit.load();
+  if (workgroups > 0) {
+    int64_t w = workgroups / kSub * kSub;  // whole chunks
+    if (w < kSub) w = kSub;
+    if (w > kGridWorkgroups) w = kGridWorkgroups;
+    launch_workgroup_limit.store(w);
+  } else if (workgroups < 0) {
+    launch_workgroup_limit.store(kGridWorkgroups);
+  }
+  return before;
 }
 
 int optimi_hip_stream_probe(optimi_group* g, int n_tensors, void* const* const* arrays, const int64_t* bytes, int n_read,

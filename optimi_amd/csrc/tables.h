@@ -53,6 +53,10 @@ struct FewTable {
 
 constexpr uint32_t bit(int i) { return 1u << i; }
 
+// One workgroup of 256 threads per tensor must fit a grid of fewer than 2^32 threads
+// (StableAdamW's per-tensor reduction).
+constexpr int kMaxTensors = (1 << 24) - 1;
+
 inline bool valid_dtype(int dtype) { return dtype == OPTIMI_F32 || dtype == OPTIMI_BF16 || dtype == OPTIMI_F16; }
 inline int elem_bytes(int dtype) { return dtype == OPTIMI_F32 ? 4 : 2; }
 inline int64_t chunk_elems(int dtype) { return kChunkBytes / elem_bytes(dtype); }
@@ -64,12 +68,12 @@ inline int64_t entry_chunk_elems(const TensorEntry& e) { return kChunkBytes / ((
 // launch does not touch (`need` has its bit clear) or that only tensors without elements would use.  `dtypes`, when not null, gives every
 // tensor's own dtype (a mixed list); otherwise all tensors have `dtype`.  Arrays in
 // `low_precision_only` (the Kahan buffer) exist for 16-bit tensors only: an fp32 tensor's
-// pointer there is ignored.  `max_chunks` bounds the launch (the grid is chunks x workgroups
-// per chunk and must fit 31 bits).  Returns an optimi_status.
+// pointer there is ignored.  `max_chunks` bounds the list (chunk numbers are kept in 32-bit
+// tables).  Returns an optimi_status.
 inline int build_entries(int n_tensors, const void* const* const* lists, int n_arrays, uint32_t need, const int64_t* numel,
                          const int* dtypes, int dtype, uint32_t low_precision_only, int64_t max_chunks, TensorEntry* out,
                          int64_t* n_chunks_out) {
-  if (n_tensors < 0) return OPTIMI_ERR_SIZE;
+  if (n_tensors < 0 || n_tensors > kMaxTensors) return OPTIMI_ERR_SIZE;
   if (!dtypes && !valid_dtype(dtype)) return OPTIMI_ERR_DTYPE;
   if (n_arrays < 0 || n_arrays > kMaxArrays) return OPTIMI_ERR_SIZE;
   if (n_tensors > 0 && (!numel || !out)) return OPTIMI_ERR_NULL;

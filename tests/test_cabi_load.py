@@ -94,3 +94,17 @@ def test_noalloc_limit_matches_its_scratch():
     for dtype, limit in ((cabi.F32, max_f32), (cabi.BF16, max_low), (cabi.F16, max_low)):
         chunk = L.optimi_hip_chunk_elems(dtype)
         assert limit % chunk == 0 and limit // chunk * 16 == partials, (dtype, limit, chunk, partials)
+
+
+def test_the_limit_is_the_grid_limit_and_rounds_to_chunks():
+    L = cabi.lib()  # no device is touched: the limit is a host-side variable
+    hardware = L.optimi_hip_launch_limit(0)
+    assert hardware == (1 << 26) - 16  # the largest whole number of chunks below 2^32 / 64 workgroups
+    try:
+        assert L.optimi_hip_launch_limit(50) == hardware
+        assert L.optimi_hip_launch_limit(1) == 48       # rounded down to whole chunks
+        assert L.optimi_hip_launch_limit(1 << 40) == 16  # at least one chunk
+        assert L.optimi_hip_launch_limit(-1) == hardware  # never above the hardware's
+        assert L.optimi_hip_launch_limit(0) == hardware
+    finally:
+        L.optimi_hip_launch_limit(-1)
