@@ -10,6 +10,8 @@
  * test suite).  All three must agree bit for bit in every buffer.  Prints one line per case and
  * "abi_host ok" at the end; exit status 1 on any mismatch or error.
  *
+ * `abi_host paths` instead walks the host side of the library (see run_paths below).
+ *
  * Build:  gcc -O1 -D__HIP_PLATFORM_AMD__ -I/opt/rocm/include -Iinclude tests/native/abi_host.c \
  *             -Loptimi_amd -loptimi_hip -Loracle -loptimi_ref -L/opt/rocm/lib -lamdhip64 -lm
  */
@@ -294,7 +296,130 @@ static int run_case(int opt, int dt) {
   return bad;
 }
 
-int main(void) {
+/* ---- "paths" mode: the library's host side walked over its own ground ----
+ * Lists that grow and shrink between 0 and 1000 tensors on one group (kernel-argument table, device
+ * tables that are rebuilt, re-uploaded or left alone, workspaces that grow), every whole-list entry
+ * point with one dtype and with a dtype per tensor, pointers that change between calls, tensors two
+ * bytes off the 16-byte grid, StableAdamW's per-tensor entry points on growing tensors, the traffic
+ * probe, the copy probe and launches split into pieces.  Results are not inspected here (the other
+ * mode and the Python tests do that): every call must succeed, and the program is meant to be run
+ * with the library's host code under AddressSanitizer as well. */
+static int64_t launches_before;
+
+static void paths_list(optimi_group* g, char* arena, size_t arena_bytes, int n, int variant) {
+  static void* ptr[MAX_ARRAYS][1000];
+  static int64_t numel[1000];
+  static int dtypes[1000];
+  size_t pos = 0;
+  for (int t = 0; t < n; ++t) {
+    numel[t] = (int64_t)(rng() % 3 == 0 ? rng() % 40 : rng() % 20000);
+    if (rng() % 11 == 0) numel[t] = 0;
+    dtypes[t] = (t % 3 == 1) ? OPTIMI_F32 : OPTIMI_BF16;
+    for (int a = 0; a < MAX_ARRAYS; ++a) {
+      size_t bytes = ((size_t)numel[t] * 4 + 15) & ~(size_t)15;
+      size_t off = (variant & 2) && a == 1 && t % 5 == 0 ? 4 : 0; /* a gradient that is a view into a bucket */
+      if (pos + bytes + 16 > arena_bytes) pos = 0;                 /* wrap: buffers may alias, values do not matter */
+      ptr[a][t] = arena + pos + off;
+      pos += bytes + 16;
+    }
+  }
+  const uint32_t f = OPTIMI_UPDATE | OPTIMI_KAHAN;
+  const void* const* gr = (const void* const*)ptr[1];
+  for (int rep = 0; rep < 2; ++rep) { /* the second time nothing has changed: no upload */
+    ABI_OK(optimi_hip_adam_multi(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[4], numel, OPTIMI_BF16, 1e-3, 0.1, 0.98, 0.02, 0.99999, 1e-6,
+                                 f | OPTIMI_DECOUPLE_WD | ((variant & 1) ? OPTIMI_RESIDENT : 0), NULL));
+  }
+  if (n > 2) { /* one gradient moves: table only */
+    void* keep = ptr[1][n / 2];
+    ptr[1][n / 2] = ptr[1][0];
+    ABI_OK(optimi_hip_adam_multi(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[4], numel, OPTIMI_BF16, 1e-3, 0.1, 0.98, 0.02, 0.0, 1e-6, f, NULL));
+    ptr[1][n / 2] = keep;
+  }
+  ABI_OK(optimi_hip_adam_multi_mixed(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[4], numel, dtypes, 1e-3, 0.1, 0.98, 0.02, 1e-2, 1e-6, f, NULL));
+  ABI_OK(optimi_hip_lion_multi(g, n, ptr[0], gr, ptr[2], ptr[3], numel, OPTIMI_F16, 1e-4, 0.1, 0.01, 0.9999, f, NULL));
+  ABI_OK(optimi_hip_lion_multi_mixed(g, n, ptr[0], gr, ptr[2], ptr[3], numel, dtypes, 1e-4, 0.1, 0.01, 0.0, OPTIMI_KAHAN, NULL));
+  ABI_OK(optimi_hip_stableadamw_multi(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[4], numel, OPTIMI_BF16, 1e-3, 0.1, 0.98, 0.02, 1e-2, 1e-6,
+                                      0.0, f, NULL));
+  ABI_OK(optimi_hip_stableadamw_multi_mixed(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[4], numel, dtypes, 1e-3, 0.1, 0.98, 0.02, 1e-2,
+                                            1e-6, 2e-3, f | OPTIMI_DECOUPLE_LR, NULL));
+  ABI_OK(optimi_hip_stableadamw_multi(g, n, ptr[0], gr, ptr[2], ptr[3], NULL, numel, OPTIMI_F32, 1e-3, 0.1, 0.98, 0.02, 1e-2, 1e-6, 0.0,
+                                      0 /* accumulate only */, NULL));
+  ABI_OK(optimi_hip_adan_multi(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[4], ptr[5], ptr[6], numel, OPTIMI_BF16, 1e-3, 0.02, 0.92, 0.08, 0.98,
+                               0.02, 1e-8, 1.00002, f, NULL));
+  ABI_OK(optimi_hip_adan_multi_mixed(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[4], ptr[5], ptr[6], numel, dtypes, 1e-3, 0.02, 0.92, 0.08,
+                                     0.98, 0.02, 1e-8, 0.99998, f | OPTIMI_ADAM_WD, NULL));
+  ABI_OK(optimi_hip_sgd_multi(g, n, ptr[0], gr, ptr[2], ptr[3], numel, OPTIMI_BF16, 1e-2, 0.9, 0.9999, f | OPTIMI_DECOUPLE_WD, NULL));
+  ABI_OK(optimi_hip_sgd_multi_mixed(g, n, ptr[0], gr, NULL, ptr[3], numel, dtypes, 1e-2, 0.0, 1e-2, f, NULL));
+  ABI_OK(optimi_hip_radam_multi(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[4], numel, OPTIMI_BF16, 1e-3, 0.1, 0.98, 0.02, 0.99999, 1e-6, 0.7,
+                                f | OPTIMI_DECOUPLE_WD | OPTIMI_RECTIFY, NULL));
+  ABI_OK(optimi_hip_radam_multi_mixed(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[4], numel, dtypes, 1e-3, 0.1, 0.98, 0.02, 0.99999, 1e-6,
+                                      0.0, f | OPTIMI_DECOUPLE_WD, NULL));
+  ABI_OK(optimi_hip_ranger_multi(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[5], ptr[4], numel, OPTIMI_BF16, 1e-3, 0.1, 0.98, 0.02, 0.99999,
+                                 1e-6, 0.7, 0.5, f | OPTIMI_DECOUPLE_WD | OPTIMI_RECTIFY | OPTIMI_LOOKAHEAD, NULL));
+  ABI_OK(optimi_hip_ranger_multi_mixed(g, n, ptr[0], gr, ptr[2], ptr[3], ptr[5], ptr[4], numel, dtypes, 1e-3, 0.1, 0.98, 0.02, 0.99999,
+                                       1e-6, 0.7, 0.5, f | OPTIMI_DECOUPLE_WD, NULL));
+  /* the traffic probe on the same tensors (sizes in bytes, multiples of 16: the aligned ones only) */
+  if (!(variant & 2) && n > 0) {
+    static int64_t bytes[1000];
+    void* const* cols[MAX_ARRAYS];
+    for (int t = 0; t < n; ++t) bytes[t] = (numel[t] * 2) & ~(int64_t)15;
+    for (int a = 0; a < MAX_ARRAYS; ++a) cols[a] = ptr[a];
+    ABI_OK(optimi_hip_stream_probe(g, n, cols, bytes, 7, 6, 0, 0, NULL));
+    ABI_OK(optimi_hip_stream_probe(g, n, cols, bytes, 3, 1, 9, OPTIMI_PROBE_SCRAMBLE, NULL));
+  }
+}
+
+static int run_paths(void) {
+  const size_t arena_bytes = (size_t)192 << 20;
+  char* arena = NULL;
+  HIP_OK(hipMalloc((void**)&arena, arena_bytes));
+  HIP_OK(hipMemset(arena, 0, arena_bytes));
+  rng_state = 1234567891234567ull;
+  optimi_group* g = NULL;
+  ABI_OK(optimi_hip_group_create(&g));
+  static const int lengths[] = {1, 16, 17, 40, 17, 300, 5, 1000, 0, 33, 2, 999, 16, 64};
+  for (size_t i = 0; i < sizeof(lengths) / sizeof(lengths[0]); ++i) {
+    if (i == 6) optimi_hip_launch_limit(48);   /* three chunks per launch from here on ... */
+    if (i == 10) optimi_hip_launch_limit(-1);  /* ... to here */
+    paths_list(g, arena, arena_bytes, lengths[i], (int)i);
+    HIP_OK(hipDeviceSynchronize());
+  }
+  /* per-tensor StableAdamW on tensors that grow and shrink (the group's partials grow), with and without a group */
+  static const int64_t sizes[] = {1, 8192, 100000, 513, 3000000, 0, 70000, 10000000, 9};
+  for (size_t i = 0; i < sizeof(sizes) / sizeof(sizes[0]); ++i) {
+    char* p = arena;
+    size_t stride = ((size_t)sizes[i] * 2 + 255) & ~(size_t)255;
+    if (6 * stride > arena_bytes) {
+      fprintf(stderr, "paths: the arena is too small for six arrays of %lld elements\n", (long long)sizes[i]);
+      return 1;
+    }
+    const uint32_t f = OPTIMI_UPDATE | OPTIMI_KAHAN;
+    ABI_OK(optimi_hip_stableadamw_single(g, p, p + stride, p + 2 * stride, p + 3 * stride, p + 4 * stride, sizes[i], OPTIMI_BF16, 1e-3,
+                                         0.1, 0.98, 0.02, 1e-2, 1e-6, 0.0, f, NULL));
+    ABI_OK(optimi_hip_stableadamw_single_noalloc(p, p + stride, p + 2 * stride, p + 3 * stride, p + 4 * stride, sizes[i], OPTIMI_F16,
+                                                 1e-3, 0.1, 0.98, 0.02, 1e-2, 1e-6, 0.0, f, NULL));
+    ABI_OK(optimi_hip_ranger_single(p, p + stride, p + 2 * stride, p + 3 * stride, p + 5 * stride, p + 4 * stride, sizes[i], OPTIMI_BF16,
+                                    1e-3, 0.1, 0.98, 0.02, 0.99999, 1e-6, 0.7, 0.5, f | OPTIMI_DECOUPLE_WD | OPTIMI_LOOKAHEAD, NULL));
+    ABI_OK(optimi_hip_radam_single(p, p + stride, p + 2 * stride, p + 3 * stride, NULL, sizes[i] / 2, OPTIMI_F32, 1e-3, 0.1, 0.98, 0.02,
+                                   0.0, 1e-6, 0.0, OPTIMI_UPDATE, NULL));
+  }
+  ABI_OK(optimi_hip_copy_probe(arena, arena + (arena_bytes >> 1), (int64_t)(arena_bytes >> 1), NULL));
+  HIP_OK(hipDeviceSynchronize());
+  /* a second group on the same lists, destroyed while the first lives on */
+  optimi_group* g2 = NULL;
+  ABI_OK(optimi_hip_group_create(&g2));
+  paths_list(g2, arena, arena_bytes, 50, 0);
+  ABI_OK(optimi_hip_group_destroy(g2));
+  paths_list(g, arena, arena_bytes, 50, 1);
+  HIP_OK(hipDeviceSynchronize());
+  ABI_OK(optimi_hip_group_destroy(g));
+  HIP_OK(hipFree(arena));
+  printf("abi_host paths ok (%lld kernels, %lld table uploads)\n", (long long)(optimi_hip_launch_count() - launches_before),
+         (long long)optimi_hip_upload_count());
+  return 0;
+}
+
+int main(int argc, char** argv) {
   int n_dev = 0;
   HIP_OK(hipGetDeviceCount(&n_dev));
   if (n_dev < 1) {
@@ -303,6 +428,10 @@ int main(void) {
   }
   HIP_OK(hipSetDevice(0));
   printf("abi version %d, %lld kernels launched so far\n", optimi_hip_version(), (long long)optimi_hip_launch_count());
+  if (argc > 1 && strcmp(argv[1], "paths") == 0) {
+    launches_before = optimi_hip_launch_count();
+    return run_paths();
+  }
   int bad = 0;
   for (int opt = 0; opt < N_OPT; ++opt) {
     bad |= run_case(opt, OPTIMI_BF16);

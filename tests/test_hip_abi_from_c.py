@@ -39,3 +39,16 @@ def test_a_plain_c_host_steps_and_matches_the_emulator(tmp_path):
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "abi_host ok" in proc.stdout, proc.stdout
     assert proc.stdout.count(": ok") == 8, proc.stdout
+
+
+@pytest.mark.gpu
+def test_the_host_side_walked_from_c(tmp_path):
+    """``abi_host paths``: lists that grow and shrink on one group, every whole-list entry point with
+    one dtype and with a dtype per tensor, moved pointers, misaligned gradients, per-tensor StableAdamW
+    on growing tensors, the probes, split launches.  Every call must succeed.  (The same program
+    with the library's host code built under AddressSanitizer and UndefinedBehaviorSanitizer is how
+    the host side was checked for memory errors; that build takes minutes and is not part of this run.)"""
+    exe = compile_host(str(tmp_path / "abi_host"))
+    proc = subprocess.run([exe, "paths"], capture_output=True, text=True, timeout=150)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "abi_host paths ok" in proc.stdout, proc.stdout
