@@ -190,8 +190,10 @@ static void check_rejections() {
   int64_t huge[2] = {INT64_MAX, INT64_MAX};
   CHECK(build_entries(2, lists, 2, 3, huge, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_ERR_SIZE, "numel that would overflow");
   int64_t at_limit[2] = {kMaxChunks * chunk_elems(OPTIMI_BF16), 1};
-  CHECK(build_entries(1, lists, 2, 3, at_limit, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_OK && n == kMaxChunks, "largest launch");
-  CHECK(build_entries(2, lists, 2, 3, at_limit, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_ERR_SIZE, "one chunk past the largest launch");
+  CHECK(build_entries(1, lists, 2, 3, at_limit, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_OK && n == kMaxChunks, "largest list");
+  CHECK(build_entries(2, lists, 2, 3, at_limit, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_ERR_SIZE, "one chunk past the largest list");
+  CHECK(build_entries(kMaxTensors + 1, lists, 2, 3, numel, nullptr, OPTIMI_BF16, 0u, kMaxChunks, out, &n) == OPTIMI_ERR_SIZE,
+        "more tensors than one workgroup each can cover in a grid");
   CHECK(build_entries(0, nullptr, 0, 0, nullptr, nullptr, OPTIMI_F32, 0u, kMaxChunks, nullptr, &n) == OPTIMI_OK && n == 0, "empty list");
   // per-tensor dtypes: each is validated, and an array that only 16-bit tensors have may be absent for fp32 ones
   const int bad_dtypes[2] = {OPTIMI_BF16, 7};
