@@ -325,7 +325,7 @@ int64_t optimi_hip_resident_launch_count(void);
 
 /* Test aid (no counterpart in the reference).  A HIP grid holds fewer than 2^32 threads, i.e.
  * fewer than 2^26 of this library's 64-lane workgroups, which is 64 GiB per array; a longer list
- * or tensor (up to 2^31 / 16 chunks of 16 KiB per array, and 2^24 - 1 tensors: OPTIMI_ERR_SIZE
+ * or tensor (up to 2^31 / 16 chunks of 16 KiB per array, and 2^22 - 1 tensors: OPTIMI_ERR_SIZE
  * beyond) is stepped by several launches, each starting where the previous one ended.  This call
  * sets the number of workgroups one launch may hold - rounded down to whole chunks (16
  * workgroups), at least one chunk, at most the hardware's limit - so that tests can run the

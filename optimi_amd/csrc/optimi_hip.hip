@@ -60,6 +60,7 @@ constexpr int kSub = kChunkBytes / (kThreads * kUnroll * 16);  // workgroups per
 static_assert(kSub >= 1 && kSub * kThreads * kUnroll * 16 == kChunkBytes, "workgroup tile must divide the chunk");
 static_assert(kThreads % 64 == 0 && kThreads <= 1024, "whole wavefronts");
 constexpr int kReduceThreads = 1024;      // lanes of the per-tensor finalize workgroup
+static_assert((int64_t)optimi_tables::kMaxTensors * kReduceThreads < ((int64_t)1 << 32), "one finalize workgroup per tensor must fit a grid");
 constexpr int kAbiVersion = 1004;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

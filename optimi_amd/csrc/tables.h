@@ -53,9 +53,9 @@ struct FewTable {
 
 constexpr uint32_t bit(int i) { return 1u << i; }
 
-// One workgroup of 256 threads per tensor must fit a grid of fewer than 2^32 threads
+// One workgroup of 1024 threads per tensor must fit a grid of fewer than 2^32 threads
 // (StableAdamW's per-tensor reduction).
-constexpr int kMaxTensors = (1 << 24) - 1;
+constexpr int kMaxTensors = (1 << 22) - 1;
 
 inline bool valid_dtype(int dtype) { return dtype == OPTIMI_F32 || dtype == OPTIMI_BF16 || dtype == OPTIMI_F16; }
 inline int elem_bytes(int dtype) { return dtype == OPTIMI_F32 ? 4 : 2; }
