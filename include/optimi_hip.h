@@ -87,8 +87,10 @@ int64_t optimi_hip_chunk_elems(int dtype);
  * Group handle.  Owns what a whole-list launch needs besides the caller's tensors:
  * the device-side tensor table (pointers, sizes), the chunk map, StableAdamW's
  * reduction partials and per-tensor scalars, and a small pinned staging ring.  None
- * of it is optimizer state; it can be dropped and rebuilt at any time.  Tables are
- * re-uploaded only when a pointer or size differs from the previous call; a list of at most
+ * of it is optimizer state; it can be dropped and rebuilt at any time.  The group keeps the
+ * tensor tables of its two most recent distinct lists on the device (gradients that alternate
+ * between two sets of buffers find theirs every time) and uploads one only when the pointers and
+ * sizes of a call match neither; the chunk map depends on the sizes alone.  A list of at most
  * 16 tensors needs no tables at all (its pointers travel as kernel arguments).  A group
  * belongs to the device that was current when it was created and must be used by
  * one thread and one stream at a time.  Under HIP graph capture a whole-list call uploads
@@ -318,7 +320,8 @@ int64_t optimi_hip_resident_bytes(void);
 
 /* Measurement aids (no counterpart in the reference), counted like optimi_hip_launch_count:
  * how many tensor tables and chunk maps have been copied to the device (a list of more than 16
- * tensors whose pointers and sizes are those of the group's previous call uploads nothing), and
+ * tensors whose pointers and sizes are those of one of the group's two most recent distinct lists
+ * uploads nothing: gradients may alternate between two sets of buffers), and
  * how many of the kernels launched for lists read their tensors with cached loads. */
 int64_t optimi_hip_upload_count(void);
 int64_t optimi_hip_resident_launch_count(void);

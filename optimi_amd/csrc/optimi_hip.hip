@@ -936,10 +936,22 @@ struct StagingSlot {
 
 }  // namespace
 
+// A tensor table on the device and the host copy of what it holds.
+struct TableSlot {
+  DeviceBuf dev;
+  std::vector<TensorEntry> host;
+  bool holds(const std::vector<TensorEntry>& fresh) const {
+    return host.size() == fresh.size() && std::memcmp(host.data(), fresh.data(), sizeof(TensorEntry) * fresh.size()) == 0;
+  }
+};
+
 struct optimi_group {
   int device = 0;
-  DeviceBuf table, chunk_map, partials, tensor_scalars;
-  std::vector<TensorEntry> host_table;   // what the device table holds
+  // Two tables: gradients that alternate between two sets of buffers (a new gradient assigned before
+  // the old one is freed, double-buffered buckets) then find their table on the device every time.
+  TableSlot tables[2];
+  int table_cur = 0;                     // the slot the last launch read
+  DeviceBuf chunk_map, partials, tensor_scalars;
   std::vector<int32_t> host_map;         // scratch for building the chunk map
   std::vector<int64_t> map_first;        // what the device chunk map was built for: every tensor's first chunk, then the chunk count
   StagingSlot ring[4];
@@ -1100,9 +1112,8 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
   // the chunk map is a function of where every tensor's chunks start and of how many there are
   bool same_map = g->map_first.size() == (size_t)n_tensors + 1 && g->map_first[(size_t)n_tensors] == n_chunks;
   for (int t = 0; same_map && t < n_tensors; ++t) same_map = g->map_first[(size_t)t] == fresh[(size_t)t].first_chunk;
-  if (capturing && ((!same_map && n_chunks > 0) ||
-                    !(g->host_table.size() == fresh.size() &&
-                      std::memcmp(g->host_table.data(), fresh.data(), sizeof(TensorEntry) * fresh.size()) == 0)))
+  int hit = g->tables[g->table_cur].holds(fresh) ? g->table_cur : g->tables[1 - g->table_cur].holds(fresh) ? 1 - g->table_cur : -1;
+  if (capturing && ((!same_map && n_chunks > 0) || hit < 0))
     return OPTIMI_ERR_CAPTURE;  // the tables must be on the device before the capture begins
   if (!same_map && n_chunks > 0) {
     g->map_first.clear();  // the cached map is void until the new one is on its way
@@ -1125,21 +1136,17 @@ int plan_list(optimi_group* g, int n_tensors, const void* const* const* lists, i
     g->map_first[(size_t)n_tensors] = n_chunks;
   }
 
-  bool same_table = g->host_table.size() == fresh.size() &&
-                    std::memcmp(g->host_table.data(), fresh.data(), sizeof(TensorEntry) * fresh.size()) == 0;
-  if (!same_table) {
-    rc = g->table.reserve(sizeof(TensorEntry) * fresh.size());
-    if (rc) {
-      g->host_table.clear();
-      return rc;
-    }
-    rc = staged_upload(g, g->table.ptr, fresh.data(), sizeof(TensorEntry) * fresh.size(), stream);
-    if (rc) {
-      g->host_table.clear();
-      return rc;
-    }
-    g->host_table.swap(fresh);
+  if (hit < 0) {  // into the slot that the last launch did not read
+    hit = 1 - g->table_cur;
+    TableSlot& slot = g->tables[hit];
+    slot.host.clear();  // void until the new table is on its way
+    rc = slot.dev.reserve(sizeof(TensorEntry) * fresh.size());
+    if (rc) return rc;
+    rc = staged_upload(g, slot.dev.ptr, fresh.data(), sizeof(TensorEntry) * fresh.size(), stream);
+    if (rc) return rc;
+    slot.host.swap(fresh);
   }
+  g->table_cur = hit;
   return 0;
 }
 
@@ -1302,7 +1309,7 @@ void launch_list(optimi_group* g, const ListPlan& plan, const typename Op::Scala
               nullptr, nullptr, plan.table, s, *s_f32, partials, first);
         else
           mixed_kernel<Op, typename Op::F32Partner, true><<<grid, dim3(kThreads), shape.lds, stream>>>(
-              (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, *s_f32, partials, first);
+              (const TensorEntry*)g->tables[g->table_cur].dev.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, *s_f32, partials, first);
         continue;
       }
     }
@@ -1310,7 +1317,7 @@ void launch_list(optimi_group* g, const ListPlan& plan, const typename Op::Scala
       step_kernel<Op, false><<<grid, dim3(kThreads), shape.lds, stream>>>(nullptr, nullptr, plan.table, s, partials, first);
     else
       step_kernel<Op, true><<<grid, dim3(kThreads), shape.lds, stream>>>(
-          (const TensorEntry*)g->table.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, partials, first);
+          (const TensorEntry*)g->tables[g->table_cur].dev.ptr, (const int32_t*)g->chunk_map.ptr, kNoTable, s, partials, first);
   }
 }
 
@@ -1568,7 +1575,7 @@ int stable_run(const ListPlan* plan, optimi_group* g, const TensorEntry& single,
           nullptr, plan->table, scratch.partials, scratch.tensor_scalars, fa);
     else
       stable_finalize_kernel<DT, true><<<dim3((unsigned)plan->n_tensors), dim3(kReduceThreads), 0, stream>>>(
-          (const TensorEntry*)g->table.ptr, kNoTable, scratch.partials, scratch.tensor_scalars, fa);
+          (const TensorEntry*)g->tables[g->table_cur].dev.ptr, kNoTable, scratch.partials, scratch.tensor_scalars, fa);
     if (kahan && wd) launch_list<StablePass2Op<DT, true, 1>>(g, *plan, s2, stream, nullptr, &s2_f32);
     else if (kahan) launch_list<StablePass2Op<DT, true, 0>>(g, *plan, s2, stream, nullptr, &s2_f32);
     else if (wd) launch_list<StablePass2Op<DT, false, 1>>(g, *plan, s2, stream, nullptr, &s2_f32);
@@ -1945,7 +1952,8 @@ int optimi_hip_group_destroy(optimi_group* g) {
     if (s.host) (void)hipHostFree(s.host);
   }
   if (g->last_launch) (void)hipEventDestroy(g->last_launch);
-  g->table.release();
+  g->tables[0].dev.release();
+  g->tables[1].dev.release();
   g->chunk_map.release();
   g->partials.release();
   g->tensor_scalars.release();

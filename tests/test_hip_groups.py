@@ -54,6 +54,43 @@ def test_each_group_keeps_its_tables_between_steps(hip_device, native):
                 G.assert_bits_equal(opt.state[p][key].cpu(), ref.state[i][key], f"{key} {i}")
 
 
+@pytest.mark.parametrize("native", [True, False], ids=["native_walk", "python_walk"])
+def test_gradients_that_alternate_between_two_sets_of_buffers_upload_nothing(hip_device, native):
+    """``p.grad = fresh_tensor`` every step makes the allocator hand out two sets of blocks in turn
+    (the new gradient exists before the old one is freed); so do double-buffered gradient buckets.
+    A group keeps two tables on the device, so once both have been seen nothing is uploaded.  Three
+    sets in rotation miss every time - results are the oracle's either way."""
+    L = cabi.lib()
+    mats, vecs = two_groups(hip_device, n_each=20)
+    params = mats + vecs
+    hyper = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=1e-2)
+    opt = optimi_amd.AdamW(params, **hyper)
+    opt.native_step = native
+    ref = ForLoopRun("adamw", [p.detach().cpu().clone() for p in params], **hyper)
+    gen = torch.Generator().manual_seed(2)
+    sets = [[(torch.randn(p.shape, generator=gen) * 1e-3).to(p.dtype) for p in params] for _ in range(3)]
+    dev_sets = [[g.to(hip_device) for g in gs] for gs in sets]
+
+    def step(k):
+        for p, g in zip(params, dev_sets[k]):
+            p.grad = g
+        before = L.optimi_hip_upload_count()
+        opt.step()
+        ref.step([g.clone() for g in sets[k]])
+        return L.optimi_hip_upload_count() - before
+
+    for it in range(4):  # set-up steps: the Python walk's first step, then both tables of the walk in use
+        step(it % 2)
+    assert [step(it % 2) for it in range(6)] == [0] * 6, "alternating gradient buffers uploaded a table again"
+    # three sets in rotation: the first of them is still on the device, after that one table (and no chunk map) per step
+    assert [step(it % 3) for it in range(1, 7)] == [0, 1, 1, 1, 1, 1]
+    torch.cuda.synchronize()
+    for i, p in enumerate(params):
+        G.assert_bits_equal(p.detach().cpu(), ref.params[i], f"param {i}")
+        for key in ("exp_avg", "exp_avg_sq", "kahan_comp"):
+            G.assert_bits_equal(opt.state[p][key].cpu(), ref.state[i][key], f"{key} {i}")
+
+
 def test_load_state_dict_and_add_param_group_drop_the_cached_tables(hip_device):
     """The workspaces are keyed by the group dicts; a state_dict round trip replaces those, and the
     tables must follow (one more upload per group, none after)."""
