@@ -980,7 +980,8 @@ class ReleaseHookCore {
 
     // pass 1: the parameters that step, their cached states (created on first sight); no side effects on steps
     struct Item {
-      at::Tensor p, g;
+      const at::Tensor* p;  // lives in the parameter list
+      at::Tensor g;         // the gradient, or a copy of it with the parameter's strides
       Entry* e;
     };
     std::vector<Item> items;
@@ -997,8 +998,8 @@ class ReleaseHookCore {
       Entry* e = find(p);
       if (!e || !valid(*e, false)) e = refresh(optimizer, k_.group_entry, py::handle(obj), p, false, group);
       at::Tensor g_like = grad_like(p, g);
-      validate_call(pack(*e, Hyper{}, p, g_like, momentum));  // everything that can reject the step, before the counter moves
-      items.push_back({p, std::move(g_like), e});
+      validate_view(view(*e, p, g_like, momentum));  // everything that can reject the step, before the counter moves
+      items.push_back({&p, std::move(g_like), e});
     }
 
     // the group's counter advances even when nothing has a gradient, as in the reference
@@ -1017,24 +1018,31 @@ class ReleaseHookCore {
     std::vector<char> done(items.size(), 0);
     for (size_t first = 0; first < items.size(); ++first) {
       if (done[first]) continue;
-      const at::Tensor& p0 = items[first].p;
+      const at::Tensor& p0 = *items[first].p;
       at::ScalarType low = at::kFloat;
       std::vector<void*> ptr[kMaxTensors];
       std::vector<char> has[kMaxTensors];  // the array exists for the tensor (a tensor without elements has no address)
       std::vector<int64_t> numel;
       std::vector<int> dtypes;
+      const size_t room = items.size() - first;
+      for (int a = 0; a < nt; ++a) {
+        ptr[a].reserve(room);
+        has[a].reserve(room);
+      }
+      numel.reserve(room);
+      dtypes.reserve(room);
       for (size_t i = first; i < items.size(); ++i) {
-        const at::Tensor& p = items[i].p;
+        const at::Tensor& p = *items[i].p;
         if (done[i] || p.device() != p0.device()) continue;
         if (p.scalar_type() != at::kFloat) {
           if (low != at::kFloat && p.scalar_type() != low) continue;
           low = p.scalar_type();
         }
         done[i] = 1;
-        const StepCall c = pack(*items[i].e, h, p, items[i].g, momentum);
+        const CallView c = view(*items[i].e, p, items[i].g, momentum);
         for (int a = 0; a < nt; ++a) {
-          ptr[a].push_back(c.t[a].has_value() ? c.t[a]->data_ptr() : nullptr);
-          has[a].push_back(c.t[a].has_value());
+          ptr[a].push_back(c.t[a] ? c.t[a]->data_ptr() : nullptr);
+          has[a].push_back(c.t[a] != nullptr);
         }
         if (p.scalar_type() == at::kFloat) ptr[nt - 1].back() = nullptr;  // no Kahan buffer for fp32
         numel.push_back(p.numel());
@@ -1207,6 +1215,37 @@ class ReleaseHookCore {
     }
     if (kind_ == SGD && momentum == 0) c.t[2] = std::nullopt;
     return c;
+  }
+
+  // The same without owning anything, for the whole-group walk: the tensors stay where they are (the
+  // parameter list, the entries' cached states, the gradients the parameters hold) for the
+  // length of the call, so pointers to them do; null = absent.
+  struct CallView {
+    const at::Tensor* t[kMaxTensors] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  };
+  CallView view(const Entry& e, const at::Tensor& p, const at::Tensor& g, double momentum) const {
+    CallView c;
+    c.t[0] = &p;
+    c.t[1] = &g;
+    const size_t n = state_keys_.size();
+    for (size_t i = 0; i < n; ++i) {
+      const std::optional<at::Tensor>& s = e.t[i];
+      if (!s.has_value()) continue;
+      const bool placeholder_possible = i + 1 == n || kind_ == SGD;  // Kahan buffer; SGD's momentum buffer
+      if (placeholder_possible && (!s->defined() || s->numel() != p.numel() || s->scalar_type() != p.scalar_type())) continue;
+      c.t[2 + i] = &*s;
+    }
+    if (kind_ == SGD && momentum == 0) c.t[2] = nullptr;
+    return c;
+  }
+  // what validate_call checks
+  void validate_view(const CallView& c) const {
+    static const char* const names[] = {"param", "grad", "state", "state", "state", "state", "state"};
+    const at::Tensor& p = *c.t[0];
+    check_param(p);
+    (void)dtype_code(p);
+    for (int a = 1; a < kTensorsOf[kind_]; ++a)
+      if (c.t[a]) check_like(p, *c.t[a], names[a]);
   }
 
   void rebind() {
