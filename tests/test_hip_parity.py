@@ -308,3 +308,28 @@ def test_copy_probe(hip_device):
     assert rc == 0
     torch.cuda.synchronize()
     assert torch.equal(src, dst)
+
+
+def test_stableadamw_gives_the_same_bits_on_every_run(hip_device):
+    """The per-tensor sum behind StableAdamW's clipped learning rate is taken in a fixed order (a
+    shuffle tree per wavefront, one partial per workgroup, the partials summed in index order by
+    one workgroup per tensor) - no atomics - so runs on the same inputs agree bit for bit however
+    the workgroups were scheduled, whole-list and per-tensor alike.  Sizes up to 20 M elements
+    (40,000 partials for the largest tensor)."""
+    from hip_engine import HipRun
+
+    hyper = CONFIGS["stableadamw"]
+    sizes = [20_000_003, 5_000_000, 70001, 8193, 513, 1] * 3  # 18 tensors: device tables
+    params, grads = draw(sizes, torch.bfloat16, 3, seed=77)
+    dev_grads = [[(g * 30).to(hip_device) for g in gs] for gs in grads]  # large gradients: the clipping is active
+
+    def run(multi):
+        r = HipRun("stableadamw", [p.to(hip_device) for p in params], multi=multi, **hyper)
+        for gs in dev_grads:
+            r.step(gs)
+        torch.cuda.synchronize()
+        return r
+
+    first = run(True)
+    for again in (run(True), run(True), run(False)):
+        G.compare_engines(first, again, "StableAdamW run to run", exact=True)
