@@ -157,10 +157,10 @@ def test_a_list_beyond_the_grid_limit(hip_device):
     group = cabi.Group()
     p = torch.ones(BEYOND, dtype=torch.bfloat16, device=hip_device)
     g = torch.ones(BEYOND, dtype=torch.bfloat16, device=hip_device)
-    # 24 tensors laid over the two buffers: 23 of a seventh of 2^26 workgroups' worth or so, ragged, and the rest
+    # 24 tensors laid over the two buffers: 23 of about 1.2 G elements each, of different sizes, and the rest
     cuts, pos = [], 0
     for i in range(23):
-        n = 8 * (150_000_000 + 12_345 * i)  # multiples of 8 elements keep every piece 16-byte aligned
+        n = 512 * (2_343_750 + 193 * i)  # multiples of 512 elements keep every piece on the 1 KiB tile grid
         cuts.append((pos, n))
         pos += n
     cuts.append((pos, BEYOND - pos))
